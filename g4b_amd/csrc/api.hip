@@ -1,0 +1,204 @@
+// C ABI of libg4b_attn.so: argument validation on the host, then dispatch to the gfx950 kernels.
+// Nothing here allocates, synchronises or reads device memory.
+#include "../../include/g4b_attn.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+
+#include "launch.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+constexpr int kDefaultWorkers = 1024;  // 256 CUs x 4 SIMDs x 1 wave
+constexpr int kMaxDecodeRows = 16;
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool dtype_ok(int dt) { return dt == G4B_DT_F16 || dt == G4B_DT_BF16 || dt == G4B_DT_F32; }
+
+uint64_t decode_slots(int B, int G, int nw) { return (uint64_t)nw + (uint64_t)B * G; }
+
+}  // namespace
+
+extern "C" {
+
+const char* g4b_last_error(void) { return g_err; }
+int32_t g4b_abi_version(void) { return G4B_ATTN_ABI_VERSION; }
+int32_t g4b_attn_default_workers(void) { return kDefaultWorkers; }
+
+uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers) {
+    if (B < 1 || H < 1 || G < 1 || Tq < 1 || D < 1 || H % G) return 0;
+    const int64_t rows = (int64_t)(H / G) * Tq;
+    if (rows > kMaxDecodeRows) return 0;
+    const int nw = num_workers > 0 ? num_workers : kDefaultWorkers;
+    return decode_slots(B, G, nw) * (uint64_t)rows * (uint64_t)(D + 2) * sizeof(float);
+}
+
+int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
+    if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
+    if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->time_dim_sizes || !a->user_phase)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, time_dim_sizes and user_phase must be non-NULL");
+    if (!dtype_ok(a->q_dtype) || !dtype_ok(a->o_dtype))
+        return fail(G4B_ERR_INVALID_ARGUMENT, "q/o dtype must be f16, bf16 or f32 (got %d, %d)", a->q_dtype, a->o_dtype);
+    if (a->kv_dtype != G4B_DT_F16 && a->kv_dtype != G4B_DT_BF16)
+        return fail(G4B_ERR_UNSUPPORTED, "KV cache dtype must be f16 or bf16 (got %d)", a->kv_dtype);
+    if (a->B < 1 || a->H < 1 || a->G < 1 || a->Tq < 1 || a->D < 1 || a->KV_CTX < 1)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "B, H, G, Tq, D, KV_CTX must be positive");
+    if (a->H % a->G) return fail(G4B_ERR_INVALID_ARGUMENT, "H (%d) must be a multiple of G (%d)", a->H, a->G);
+    if (a->D != 128 && a->D != 256) return fail(G4B_ERR_UNSUPPORTED, "head_dim %d not built (128 and 256 are)", a->D);
+    if (a->B > 65535 || a->G > 65535) return fail(G4B_ERR_UNSUPPORTED, "B and G must be <= 65535");
+    if (a->ctx_window_size < 1 || a->ctx_window_size > a->KV_CTX)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "ctx_window_size (%d) must be in [1, KV_CTX = %d]", a->ctx_window_size, a->KV_CTX);
+    if (a->stage == G4B_STAGE_ON_BAND)
+        return fail(G4B_ERR_UNSUPPORTED, "STAGE_ON_BAND alone depends on the reference's tile size and is not built");
+    if (a->stage != G4B_STAGE_FULL && a->stage != G4B_STAGE_CAUSAL)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "stage must be STAGE_FULL (1) or STAGE_CAUSAL (3), got %d", a->stage);
+    if (a->phase < 0 || a->phase > 255) return fail(G4B_ERR_INVALID_ARGUMENT, "phase must fit uint8");
+    if (a->query_window < 0) return fail(G4B_ERR_INVALID_ARGUMENT, "query_window must be >= 0");
+    if (!std::isfinite(a->scale)) return fail(G4B_ERR_INVALID_ARGUMENT, "scale must be finite");
+    if (a->q_stride[3] != 1 || a->o_stride[3] != 1)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "q and o must have unit stride in the head dimension");
+    for (int i = 0; i < 3; ++i)
+        if (a->q_stride[i] % 8 || a->o_stride[i] % 8)
+            return fail(G4B_ERR_INVALID_ARGUMENT, "q/o strides must be multiples of 8 elements (16-byte vector access)");
+    if (!aligned16(a->q) || !aligned16(a->o) || !aligned16(a->k_cache) || !aligned16(a->v_cache))
+        return fail(G4B_ERR_INVALID_ARGUMENT, "q, o, k_cache, v_cache must be 16-byte aligned");
+    const int64_t slot_elems = (int64_t)a->G * a->KV_CTX * a->D;
+    if (a->k_stride_b < slot_elems || a->v_stride_b < slot_elems || a->k_stride_b % 8 || a->v_stride_b % 8)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "cache slot stride must be >= G*KV_CTX*D and a multiple of 8 elements");
+    if ((int64_t)a->KV_CTX * a->D * 2 >= (int64_t)1 << 31)
+        return fail(G4B_ERR_UNSUPPORTED, "KV_CTX * D * 2 bytes must be below 2 GiB per (slot, kv head)");
+    if (a->num_workers < 0 || a->num_workers > (1 << 20)) return fail(G4B_ERR_INVALID_ARGUMENT, "num_workers out of range");
+
+    g4b::AttnParams p{};
+    p.q = a->q;
+    p.k = a->k_cache;
+    p.v = a->v_cache;
+    p.o = a->o;
+    p.tds = a->time_dim_sizes;
+    p.phase_arr = a->user_phase;
+    p.win_arr = a->window_sizes;
+    for (int i = 0; i < 4; ++i) {
+        p.q_s[i] = a->q_stride[i];
+        p.o_s[i] = a->o_stride[i];
+    }
+    p.k_sb = a->k_stride_b;
+    p.v_sb = a->v_stride_b;
+    p.tds_s = a->time_dim_sizes_stride;
+    p.ph_s = a->user_phase_stride;
+    p.win_s = a->window_sizes_stride;
+    p.q_dt = a->q_dtype;
+    p.o_dt = a->o_dtype;
+    p.B = a->B;
+    p.H = a->H;
+    p.G = a->G;
+    p.R = a->H / a->G;
+    p.Tq = a->Tq;
+    p.KV_CTX = a->KV_CTX;
+    p.W = a->ctx_window_size;
+    p.phase = a->phase;
+    p.stage = a->stage;
+    p.qwin = a->query_window;
+    p.c = a->scale * 1.44269504088896340736f;
+
+    const int64_t rows = (int64_t)p.R * p.Tq;
+    hipError_t e;
+    if (rows <= kMaxDecodeRows) {
+        if (a->workspace) {
+            const int nw = a->num_workers > 0 ? a->num_workers : kDefaultWorkers;
+            const uint64_t need = g4b_attn_workspace_bytes(a->B, a->H, a->G, a->Tq, a->D, nw);
+            if (a->workspace_bytes < need)
+                return fail(G4B_ERR_WORKSPACE, "workspace holds %llu bytes, %llu needed for %d workers",
+                            (unsigned long long)a->workspace_bytes, (unsigned long long)need, nw);
+            if (!aligned16(a->workspace)) return fail(G4B_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+            p.NW = nw;
+            p.part_o = static_cast<float*>(a->workspace);
+            p.part_ml = p.part_o + decode_slots(a->B, a->G, nw) * (uint64_t)rows * (uint64_t)a->D;
+        } else {
+            p.NW = 0;  // one wave per (slot, kv head), no partials
+        }
+        e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
+    } else {
+        if (128 % p.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide 128 for prefill-shaped launches", p.R);
+        e = g4b::launch_attn_prefill(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
+    }
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
+int g4b_kv_append(const g4b_kv_append_args* a, void* stream) {
+    if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
+    if (!a->x || !a->cache || !a->cache_offsets) return fail(G4B_ERR_INVALID_ARGUMENT, "x, cache and cache_offsets must be non-NULL");
+    if (!dtype_ok(a->x_dtype) || !dtype_ok(a->cache_dtype)) return fail(G4B_ERR_INVALID_ARGUMENT, "x/cache dtype must be f16, bf16 or f32");
+    if (a->B < 1 || a->G < 1 || a->t < 1 || a->T < 1 || a->D < 1) return fail(G4B_ERR_INVALID_ARGUMENT, "B, G, t, T, D must be positive");
+    if (a->t > a->T) return fail(G4B_ERR_INVALID_ARGUMENT, "t (%d) must not exceed the ring length T (%d)", a->t, a->T);
+    if (a->D % 8) return fail(G4B_ERR_UNSUPPORTED, "D must be a multiple of 8");
+    if (a->B > 65535) return fail(G4B_ERR_UNSUPPORTED, "B must be <= 65535");
+    if (a->phase < 0 || a->phase > 255) return fail(G4B_ERR_INVALID_ARGUMENT, "phase must fit uint8");
+    if (a->x_stride[3] != 1) return fail(G4B_ERR_INVALID_ARGUMENT, "x must have unit stride in the head dimension");
+    for (int i = 0; i < 3; ++i)
+        if (a->x_stride[i] % 8) return fail(G4B_ERR_INVALID_ARGUMENT, "x strides must be multiples of 8 elements");
+    if (a->cache_stride_b < (int64_t)a->G * a->T * a->D || a->cache_stride_b % 8)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "cache slot stride must be >= G*T*D and a multiple of 8 elements");
+    if (!aligned16(a->x) || !aligned16(a->cache)) return fail(G4B_ERR_INVALID_ARGUMENT, "x and cache must be 16-byte aligned");
+    if (!std::isfinite(a->rmsnorm_eps)) return fail(G4B_ERR_INVALID_ARGUMENT, "rmsnorm_eps must be finite");
+
+    g4b::KvAppendParams p{};
+    p.x = a->x;
+    p.cache = a->cache;
+    p.offsets = a->cache_offsets;
+    p.x_rsos = a->x_rsos;
+    p.phase_arr = a->user_phase;
+    for (int i = 0; i < 4; ++i) p.x_s[i] = a->x_stride[i];
+    for (int i = 0; i < 3; ++i) p.rsos_s[i] = a->x_rsos_stride[i];
+    p.cache_sb = a->cache_stride_b;
+    p.off_s = a->cache_offsets_stride;
+    p.ph_s = a->user_phase_stride;
+    p.x_dt = a->x_dtype;
+    p.cache_dt = a->cache_dtype;
+    p.off_is_i64 = a->cache_offsets_is_int64 ? 1 : 0;
+    p.B = a->B;
+    p.G = a->G;
+    p.t = a->t;
+    p.T = a->T;
+    p.D = a->D;
+    p.phase = a->phase;
+    p.eps = a->rmsnorm_eps;
+    hipError_t e = g4b::launch_kv_append(p, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "kv append launch failed: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
+int g4b_advance_decode_state(const g4b_advance_args* a, void* stream) {
+    if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
+    if (!a->input_token_ids || !a->out_token_ids || !a->cache_offsets || !a->time_dim_sizes || !a->user_phase)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "all five arrays must be non-NULL");
+    if (a->B < 1) return fail(G4B_ERR_INVALID_ARGUMENT, "B must be positive");
+    g4b::AdvanceParams p{};
+    p.input_token_ids = a->input_token_ids;
+    p.out_token_ids = a->out_token_ids;
+    p.cache_offsets = a->cache_offsets;
+    p.time_dim_sizes = a->time_dim_sizes;
+    p.user_phase = a->user_phase;
+    p.in_s1 = a->input_token_ids_stride1;
+    p.out_s0 = a->out_token_ids_stride0;
+    p.off_s = a->cache_offsets_stride;
+    p.tds_s = a->time_dim_sizes_stride;
+    p.ph_s = a->user_phase_stride;
+    p.B = a->B;
+    hipError_t e = g4b::launch_advance_decode_state(p, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "advance launch failed: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,388 @@
+// Decode attention for gfx950: the query block of one (slot, kv head) pair is at most 16 rows
+// (R = H/G heads x Tq tokens), the KV cache is streamed from HBM exactly once per pair.
+//
+// Work decomposition.  Every in-phase slot contributes ceil(keys / 32) tiles per kv head; the
+// tiles of all pairs form one flat list that is dealt evenly to NW single-wave workgroups
+// (worker w owns flat tiles [w*T/NW, (w+1)*T/NW)).  The split is computed on the device from
+// time_dim_sizes, so the grid is static while the balance follows the real lengths.  A worker
+// whose range covers a whole pair writes the output directly; otherwise it leaves an
+// un-normalised fp32 partial (acc, running max, running sum) in workspace slot (w + pair) and a
+// second kernel merges the partials of each pair.
+//
+// Tile math (one wave, 32 keys).  S^T = K Q^T and O^T += V^T P run on v_mfma_f32_16x16x32.
+// The 16 output columns carry (row, class) pairs: the D/8 16-byte pieces of a key row are dealt
+// round-robin to CL classes, lane quad members read neighbouring pieces (64 contiguous bytes per
+// quad, 256 per key row and instruction), and the diagonal (class == class) blocks of the MFMA
+// result summed over the CL lanes of a row give the dot product.  P stays in registers: the
+// score layout of the first MFMA is the B-operand layout of the second, with the key order of the
+// contraction chosen to match.  V^T operands are built with an in-lane 8x8 16-bit transpose.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace g4b {
+
+constexpr int DEC_TILE = 32;  // keys per wave iteration
+
+G4B_DEV int slot_tiles(const AttnParams& p, int b) {
+    SlotInfo s = slot_info(p, b);
+    return (s.window - s.klo + DEC_TILE - 1) / DEC_TILE;
+}
+
+template <int CL>
+G4B_DEV float pick(const f4& c, int e, int cls) {
+    // element e*CL + cls of c without dynamic register indexing
+    if constexpr (CL == 1) {
+        return c[e];
+    } else if constexpr (CL == 2) {
+        return cls ? c[2 * e + 1] : c[2 * e];
+    } else {
+        float lo = (cls & 1) ? c[1] : c[0];
+        float hi = (cls & 1) ? c[3] : c[2];
+        return (cls & 2) ? hi : lo;
+    }
+}
+
+// One segment: tiles [t0, t1) of pair (bb, g) whose slot has tlb tiles per kv head.  Worker w
+// writes the output itself when the segment is the whole pair, else partial slot (w + pair).
+template <int D, int CL, class T>
+G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb) {
+    constexpr int E = 4 / CL;          // scores a lane keeps per 16-row MFMA tile
+    constexpr int KT = 16 / CL;        // keys per MFMA tile
+    constexpr int NT = DEC_TILE / KT;  // MFMA tiles per 32 keys
+    constexpr int PIECES = D / 8;      // 16-byte pieces per key row
+    constexpr int NC = PIECES / (4 * CL);
+    constexpr int DC = D / 128;
+    constexpr int ROWB = D * 2;  // bytes per cache row
+    static_assert(NC >= 1 && DC >= 1, "head dim too small for this tiling");
+    const int lane = threadIdx.x;
+    const int m16 = lane & 15, g4 = lane >> 4;
+    const int cls = m16 % CL;
+    const int G = p.G, Tq = p.Tq;
+    const int NR = p.R * Tq;
+
+    const SlotInfo si = slot_info(p, bb);
+    const int KV_CTX = p.KV_CTX;
+    const char* kbase =
+        static_cast<const char*>(p.k) + ((int64_t)bb * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
+    const char* vbase =
+        static_cast<const char*>(p.v) + ((int64_t)bb * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
+
+    // this lane's query row (as MFMA column n = m16 = row*CL + cls)
+    const int row = m16 / CL;
+    const bool row_ok = row < NR;
+    const int hh = row_ok ? row / Tq : 0;
+    const int ti = row_ok ? row % Tq : 0;
+    int lo_r, hi_r;
+    row_range(p, si, ti, lo_r, hi_r);
+    int lo_max, hi_min, dummy;
+    row_range(p, si, Tq - 1, lo_max, dummy);
+    row_range(p, si, 0, dummy, hi_min);
+
+    u4 qf[NC];
+    {
+        const int64_t qoff = (int64_t)bb * p.q_s[0] + (int64_t)(g * p.R + hh) * p.q_s[1] + (int64_t)ti * p.q_s[2];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int piece = cls + CL * g4 + 4 * CL * c;
+            u4 z = {0, 0, 0, 0};
+            qf[c] = row_ok ? load8_as<T>(p.q, qoff + piece * 8, p.q_dt) : z;
+        }
+    }
+
+    // byte offset of (logical key j, 16-byte piece) in the ring; j clamped to the window
+    auto key_off = [&](int j) -> uint32_t {
+        j = min(j, si.window - 1);
+        int r = si.ring_start + j;
+        r = (r >= KV_CTX) ? r - KV_CTX : r;
+        return (uint32_t)r * ROWB;
+    };
+
+    u4 kreg[NT][NC];
+    u4 vreg[DC][8];
+    auto load_k = [&](int t) {
+        const int jb = si.klo + t * DEC_TILE;
+#pragma unroll
+        for (int tau = 0; tau < NT; ++tau) {
+            const uint32_t ro = key_off(jb + tau * KT + m16 / CL);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) kreg[tau][c] = ld16(kbase, ro + (uint32_t)(cls + CL * g4 + 4 * CL * c) * 16u);
+        }
+    };
+    auto load_v = [&](int t) {
+        const int jb = si.klo + t * DEC_TILE;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint32_t ro = key_off(jb + (s / E) * KT + g4 * E + (s % E));
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) vreg[dc][s] = ld16(vbase, ro + (uint32_t)(m16 + 16 * dc) * 16u);
+        }
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f4 acc[DC * 8];
+#pragma unroll
+    for (int i = 0; i < DC * 8; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+
+    load_k(t0);
+    load_v(t0);
+    for (int t = t0; t < t1; ++t) {
+        const int jb = si.klo + t * DEC_TILE;
+        // ---- S^T = K Q^T -------------------------------------------------------
+        float sc[8];
+#pragma unroll
+        for (int tau = 0; tau < NT; ++tau) {
+            f4 c4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NC; ++c) c4 = T::mfma16(kreg[tau][c], qf[c], c4);
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float x = pick<CL>(c4, e, cls);
+                if constexpr (CL >= 2) x += quad_xor1(x);
+                if constexpr (CL == 4) x += quad_xor2(x);
+                sc[tau * E + e] = x * p.c;
+            }
+        }
+        if (t + 1 < t1) load_k(t + 1);
+
+        // ---- online softmax (per row; a row's keys are spread over the 4 lane groups)
+        if (jb < lo_max || jb + DEC_TILE > hi_min) {
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const int j = jb + (s / E) * KT + g4 * E + (s % E);
+                if (j < lo_r || j >= hi_r) sc[s] = -INFINITY;
+            }
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int s = 1; s < 8; ++s) mx = fmaxf(mx, sc[s]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        float ps[8], psum = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            ps[s] = fast_exp2(sc[s] - m_safe);
+            psum += ps[s];
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        const u4 pf = {T::pack2(ps[0], ps[1]), T::pack2(ps[2], ps[3]), T::pack2(ps[4], ps[5]), T::pack2(ps[6], ps[7])};
+#pragma unroll
+        for (int i = 0; i < DC * 8; ++i) acc[i] *= alpha;
+
+        // ---- O^T += V^T P ------------------------------------------------------
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+            u4 vt[8];
+            transpose8x8_b16(vreg[dc], vt);
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) acc[dc * 8 + jj] = T::mfma16(vt[jj], pf, acc[dc * 8 + jj]);
+        }
+        if (t + 1 < t1) load_v(t + 1);
+    }
+
+    // ---- epilogue -----------------------------------------------------------------
+    float l_tot = l_run + __shfl_xor(l_run, 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    const bool whole = (t0 == 0 && t1 == tlb);
+    if (row_ok) {
+        if (whole) {
+            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+            const int64_t ooff =
+                (int64_t)bb * p.o_s[0] + (int64_t)(g * p.R + hh) * p.o_s[1] + (int64_t)ti * p.o_s[2];
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    float v8[8];
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj) v8[jj] = pick<CL>(acc[dc * 8 + jj], e, cls) * inv;
+                    const int d0 = 128 * dc + (4 * g4 + e * CL + cls) * 8;
+                    store8(p.o, ooff + d0, p.o_dt, v8);
+                }
+            }
+        } else {
+            const int64_t slot = (int64_t)w + (int64_t)bb * G + g;
+            float* po = p.part_o + (slot * NR + row) * D;
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    float v8[8];
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj) v8[jj] = pick<CL>(acc[dc * 8 + jj], e, cls);
+                    const int d0 = 128 * dc + (4 * g4 + e * CL + cls) * 8;
+                    store8(po, d0, DT_F32, v8);
+                }
+            }
+            if (cls == 0 && g4 == 0) {
+                float* pm = p.part_ml + (slot * NR + row) * 2;
+                pm[0] = m_run;
+                pm[1] = l_tot;
+            }
+        }
+    }
+}
+
+template <int D, int CL, class T>
+__global__ __launch_bounds__(64, 1) void attn_decode_worker(const AttnParams p) {
+    const int lane = threadIdx.x;
+    const int w = blockIdx.x;
+    const int B = p.B, G = p.G;
+
+    if (p.NW == 0) {
+        // no workspace: worker w owns the whole pair w
+        const int bb = w / G, g = w % G;
+        const int tlb = slot_tiles(p, bb);
+        if (tlb > 0) decode_segment<D, CL, T>(p, w, bb, g, 0, tlb, tlb);
+        return;
+    }
+
+    // ---- flat tile list: total, then this worker's range ------------------------------------
+    int total = 0;
+    for (int b0 = 0; b0 < B; b0 += 64) {
+        int b = b0 + lane;
+        total += (b < B) ? G * slot_tiles(p, b) : 0;
+    }
+    total = wave_sum_i(total);
+    const int nw = min(p.NW, total);  // never more workers than tiles: every worker below nw owns >= 1 tile
+    if (w >= nw) return;
+    const int64_t ws = (int64_t)w * total / nw;
+    const int64_t we = (int64_t)(w + 1) * total / nw;
+
+    int carry = 0;
+    for (int b0 = 0; b0 < B; b0 += 64) {
+        const int bl = b0 + lane;
+        const int tl = (bl < B) ? slot_tiles(p, bl) : 0;
+        const int cnt = G * tl;
+        const int incl = wave_incl_scan_i(cnt, lane);
+        const int excl = carry + incl - cnt;
+        const bool hit = cnt > 0 && (int64_t)excl < we && (int64_t)excl + cnt > ws;
+        uint64_t mask = __ballot(hit);
+        while (mask) {
+            const int src = __builtin_ctzll(mask);
+            mask &= mask - 1;
+            const int bb = b0 + src;
+            const int ex = __shfl(excl, src);
+            const int tlb = __shfl(tl, src);
+            for (int g = 0; g < G; ++g) {
+                const int64_t fs = (int64_t)ex + (int64_t)g * tlb;
+                const int t0 = (int)(max(ws, fs) - fs);
+                const int t1 = (int)(min(we, fs + tlb) - fs);
+                if (t1 > t0) decode_segment<D, CL, T>(p, w, bb, g, t0, t1, tlb);
+            }
+        }
+        carry += __shfl(incl, 63);
+        if ((int64_t)carry >= we) break;
+    }
+}
+
+// Merge the partials of each (slot, kv head) pair; one workgroup per pair, 256 threads.
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
+    __shared__ int red[256];
+    const int tid = threadIdx.x;
+    const int pair = blockIdx.x;
+    const int b = pair / p.G, g = pair % p.G;
+    const int B = p.B, G = p.G;
+    const int NR = p.R * p.Tq;
+
+    // flat start of this pair and total tile count (same arithmetic as the workers)
+    int before = 0, total = 0;
+    for (int x = tid; x < B; x += 256) {
+        int c = G * slot_tiles(p, x);
+        total += c;
+        if (x < b) before += c;
+    }
+    red[tid] = before;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o) red[tid] += red[tid + o];
+        __syncthreads();
+    }
+    before = red[0];
+    __syncthreads();
+    red[tid] = total;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o) red[tid] += red[tid + o];
+        __syncthreads();
+    }
+    total = red[0];
+
+    const SlotInfo si = slot_info(p, b);
+    if (!si.active) return;
+    const int tl = slot_tiles(p, b);
+    const int nvec = NR * (D / 4);
+    if (tl == 0) {
+        // in-phase slot without any visible key: defined as zeros
+        for (int x = tid; x < nvec; x += 256) {
+            const int row = x / (D / 4), d0 = (x % (D / 4)) * 4;
+            const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] +
+                                 (int64_t)(row % p.Tq) * p.o_s[2] + d0;
+            store4(p.o, ooff, p.o_dt, f4{0.f, 0.f, 0.f, 0.f});
+        }
+        return;
+    }
+    if (p.NW == 0) return;  // one wave owned the whole pair
+    const int nw = min(p.NW, total);
+    const int64_t fs = (int64_t)before + (int64_t)g * tl;
+    // worker that owns flat tile x: the largest w with floor(w * total / nw) <= x
+    const int w0 = (int)(((fs + 1) * nw - 1) / total);
+    const int w1 = (int)(((fs + tl) * nw - 1) / total);
+    if (w0 == w1) return;  // a single worker owned the pair and wrote the output itself
+
+    for (int x = tid; x < nvec; x += 256) {
+        const int row = x / (D / 4), d0 = (x % (D / 4)) * 4;
+        float m = -INFINITY, l = 0.f;
+        f4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int w = w0; w <= w1; ++w) {
+            const int64_t slot = (int64_t)w + pair;
+            const float* pm = p.part_ml + (slot * NR + row) * 2;
+            const float mw = pm[0], lw = pm[1];
+            if (mw == -INFINITY) continue;
+            const f4 ow = *reinterpret_cast<const f4*>(p.part_o + (slot * NR + row) * D + d0);
+            const float mn = fmaxf(m, mw);
+            const float a = fast_exp2(m - mn), bw = fast_exp2(mw - mn);
+            acc = acc * a + ow * bw;
+            l = l * a + lw * bw;
+            m = mn;
+        }
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] +
+                             (int64_t)(row % p.Tq) * p.o_s[2] + d0;
+        store4(p.o, ooff, p.o_dt, acc * inv);
+    }
+}
+
+template <int D, int CL, class T>
+static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
+    hipLaunchKernelGGL((attn_decode_worker<D, CL, T>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <int D, class T>
+static hipError_t launch_decode_cl(const AttnParams& p, hipStream_t stream) {
+    const int rows = p.R * p.Tq;
+    if (rows <= 4) return launch_decode_t<D, 4, T>(p, stream);
+    if (rows <= 8) return launch_decode_t<D, 2, T>(p, stream);
+    return launch_decode_t<D, 1, T>(p, stream);
+}
+
+hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream) {
+    if (kv_dt == DT_F16) {
+        if (D == 256) return launch_decode_cl<256, F16>(p, stream);
+        if (D == 128) return launch_decode_cl<128, F16>(p, stream);
+    } else {
+        if (D == 256) return launch_decode_cl<256, BF16>(p, stream);
+        if (D == 128) return launch_decode_cl<128, BF16>(p, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace g4b

@@ -1,0 +1,206 @@
+// Shared device helpers for the gfx950 attention kernels: vector types, MFMA wrappers for
+// fp16 / bf16 operands, 16-byte global loads, wave64 cross-lane primitives, and the per-slot
+// window arithmetic every kernel evaluates the same way.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace g4b {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2 };
+enum : int { STAGE_FULL = 1, STAGE_ON_BAND = 2, STAGE_CAUSAL = 3 };
+
+#define G4B_DEV __device__ __forceinline__
+
+// ---- element types of the KV cache (and of the MFMA operands) ---------------------------------
+struct F16 {
+    static constexpr int dt = DT_F16;
+    static G4B_DEV f4 mfma16(u4 a, u4 b, f4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    }
+    static G4B_DEV f16v mfma32(u4 a, u4 b, f16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    }
+    static G4B_DEV uint32_t pack2(float lo, float hi) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static G4B_DEV float lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); }
+    static G4B_DEV float hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
+};
+
+struct BF16 {
+    static constexpr int dt = DT_BF16;
+    static G4B_DEV f4 mfma16(u4 a, u4 b, f4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    }
+    static G4B_DEV f16v mfma32(u4 a, u4 b, f16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, a), __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    }
+    static G4B_DEV uint32_t pack2(float lo, float hi) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        b2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static G4B_DEV float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+    static G4B_DEV float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+};
+
+// ---- memory ----------------------------------------------------------------------------------
+G4B_DEV u4 ld16(const void* base, uint32_t byte_off) {
+    return *reinterpret_cast<const u4*>(static_cast<const char*>(base) + byte_off);
+}
+G4B_DEV u4 ld16(const void* base, int64_t byte_off) {
+    return *reinterpret_cast<const u4*>(static_cast<const char*>(base) + byte_off);
+}
+
+// Eight consecutive elements of a q/x row (dtype chosen at run time) as eight MFMA operand
+// elements of type T, optionally pre-multiplied.
+template <class T>
+G4B_DEV u4 load8_as(const void* base, int64_t elem_off, int dt) {
+    if (dt == DT_F32) {
+        const f4* p = reinterpret_cast<const f4*>(static_cast<const float*>(base) + elem_off);
+        f4 a = p[0], b = p[1];
+        u4 r = {T::pack2(a[0], a[1]), T::pack2(a[2], a[3]), T::pack2(b[0], b[1]), T::pack2(b[2], b[3])};
+        return r;
+    }
+    u4 raw = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off);
+    if (dt == T::dt) return raw;
+    u4 r;
+    if (dt == DT_F16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = T::pack2(F16::lo(raw[i]), F16::hi(raw[i]));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = T::pack2(BF16::lo(raw[i]), BF16::hi(raw[i]));
+    }
+    return r;
+}
+
+// Store eight consecutive output elements (dtype chosen at run time) from eight floats.
+G4B_DEV void store8(void* base, int64_t elem_off, int dt, const float (&v)[8]) {
+    if (dt == DT_F32) {
+        f4* p = reinterpret_cast<f4*>(static_cast<float*>(base) + elem_off);
+        f4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+        p[0] = a;
+        p[1] = b;
+    } else if (dt == DT_F16) {
+        u4 r = {F16::pack2(v[0], v[1]), F16::pack2(v[2], v[3]), F16::pack2(v[4], v[5]), F16::pack2(v[6], v[7])};
+        *reinterpret_cast<u4*>(static_cast<uint16_t*>(base) + elem_off) = r;
+    } else {
+        u4 r = {BF16::pack2(v[0], v[1]), BF16::pack2(v[2], v[3]), BF16::pack2(v[4], v[5]), BF16::pack2(v[6], v[7])};
+        *reinterpret_cast<u4*>(static_cast<uint16_t*>(base) + elem_off) = r;
+    }
+}
+
+G4B_DEV void store4(void* base, int64_t elem_off, int dt, f4 v) {
+    if (dt == DT_F32) {
+        *reinterpret_cast<f4*>(static_cast<float*>(base) + elem_off) = v;
+    } else if (dt == DT_F16) {
+        u2 r = {F16::pack2(v[0], v[1]), F16::pack2(v[2], v[3])};
+        *reinterpret_cast<u2*>(static_cast<uint16_t*>(base) + elem_off) = r;
+    } else {
+        u2 r = {BF16::pack2(v[0], v[1]), BF16::pack2(v[2], v[3])};
+        *reinterpret_cast<u2*>(static_cast<uint16_t*>(base) + elem_off) = r;
+    }
+}
+
+// ---- wave64 cross-lane -----------------------------------------------------------------------
+template <int CTRL>
+G4B_DEV float dpp_f(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+G4B_DEV float quad_xor1(float x) { return dpp_f<0xB1>(x); }  // quad_perm [1,0,3,2]
+G4B_DEV float quad_xor2(float x) { return dpp_f<0x4E>(x); }  // quad_perm [2,3,0,1]
+
+G4B_DEV int wave_sum_i(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+G4B_DEV int wave_incl_scan_i(int v, int lane) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int t = __shfl_up(v, o);
+        if (lane >= o) v += t;
+    }
+    return v;
+}
+
+G4B_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// In-lane 8x8 transpose of 16-bit elements.  in[s] holds elements (s, 0..7); out[j] holds (0..7, j).
+G4B_DEV void transpose8x8_b16(const u4 (&in)[8], u4 (&out)[8]) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            uint32_t a = in[2 * t][w], b = in[2 * t + 1][w];
+            out[2 * w][t] = __builtin_amdgcn_perm(b, a, 0x05040100u);      // low halves:  a.lo | b.lo << 16
+            out[2 * w + 1][t] = __builtin_amdgcn_perm(b, a, 0x07060302u);  // high halves: a.hi | b.hi << 16
+        }
+    }
+}
+
+// ---- launch parameters shared by the attention kernels -----------------------------------------
+struct AttnParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    const int32_t* tds;
+    const uint8_t* phase_arr;
+    const int32_t* win_arr;  // optional per-slot window sizes
+    float* part_o;           // split partials: [slot][row][D] un-normalised fp32
+    float* part_ml;          // [slot][row][2] = (running max in log2 units, running sum)
+    int64_t q_s[4], o_s[4];  // element strides of q and o ([B,H,Tq,D])
+    int64_t k_sb, v_sb;      // batch strides of the caches (elements)
+    int64_t tds_s, ph_s, win_s;
+    int32_t q_dt, o_dt;
+    int32_t B, H, G, R, Tq, KV_CTX;
+    int32_t W, phase, stage, qwin;
+    int32_t NW;  // number of decode workers (waves) the key tiles are dealt to
+    float c;     // softmax scale * log2(e)
+};
+
+// What an attention launch reads of one slot.  window = min(tds, W) keys ending at the newest
+// token; logical key j sits in ring row (ring_start + j) mod KV_CTX; query i is aligned with
+// logical key qb + i.  [klo, window) is the union of the key ranges of all queries of the launch.
+struct SlotInfo {
+    int window, ring_start, qb, klo;
+    bool active;
+};
+
+G4B_DEV SlotInfo slot_info(const AttnParams& p, int b) {
+    SlotInfo s;
+    s.active = p.phase_arr[(int64_t)b * p.ph_s] == (uint8_t)p.phase;
+    int tds = p.tds[(int64_t)b * p.tds_s];
+    int W = p.win_arr ? p.win_arr[(int64_t)b * p.win_s] : p.W;
+    W = min(max(W, 0), p.KV_CTX);
+    tds = max(tds, 0);
+    s.window = s.active ? min(tds, W) : 0;
+    int base = tds - min(tds, W);
+    s.ring_start = base % p.KV_CTX;
+    s.qb = s.window - p.Tq;
+    int klo = 0;
+    if (p.qwin > 0) klo = min(max(0, s.qb - p.qwin + 1), s.window);
+    s.klo = klo;
+    return s;
+}
+
+// Visible logical key range [lo, hi) of query i of a slot.
+G4B_DEV void row_range(const AttnParams& p, const SlotInfo& s, int i, int& lo, int& hi) {
+    int qp = s.qb + i;
+    hi = (p.stage == STAGE_FULL) ? s.window : min(s.window, qp + 1);
+    lo = (p.qwin > 0) ? max(0, qp - p.qwin + 1) : 0;
+}
+
+}  // namespace g4b

@@ -1,0 +1,43 @@
+// Host-side launchers implemented by the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "common.hpp"
+
+namespace g4b {
+
+// rows = (H/G) * Tq <= 16, D in {128, 256}; kv_dt in {DT_F16, DT_BF16}
+hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
+// any Tq; (H/G) must divide 128
+hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
+
+struct KvAppendParams {
+    const void* x;
+    void* cache;
+    const void* offsets;    // int32 or int64
+    const float* x_rsos;    // optional [B,G,t] row sums of squares
+    const uint8_t* phase_arr;  // optional
+    int64_t x_s[4];
+    int64_t rsos_s[3];
+    int64_t cache_sb;  // batch stride of the cache (elements)
+    int64_t off_s, ph_s;
+    int32_t x_dt, cache_dt, off_is_i64;
+    int32_t B, G, t, T, D;
+    int32_t phase;
+    float eps;
+};
+hipError_t launch_kv_append(const KvAppendParams& p, hipStream_t stream);
+
+struct AdvanceParams {
+    int32_t* input_token_ids;  // [t, B], row 0 written
+    const int32_t* out_token_ids;  // [B, >=1], column 0 read
+    int32_t* cache_offsets;
+    int32_t* time_dim_sizes;
+    const uint8_t* user_phase;
+    int64_t in_s1, out_s0, off_s, tds_s, ph_s;
+    int32_t B;
+};
+hipError_t launch_advance_decode_state(const AdvanceParams& p, hipStream_t stream);
+
+}  // namespace g4b

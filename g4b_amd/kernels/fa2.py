@@ -1,0 +1,183 @@
+"""Flash attention over the per-slot ring KV cache -- drop-in for ``g4b/kernels/fa2.py``.
+
+Same public surface as the reference module: the ``STAGE_*`` / ``PHASE_*`` constants
+(``fa2.py:14-34``) and :func:`flash_attention` with the reference's positional signature
+(``fa2.py:634-652``).  The work is done by ``g4b_attn_forward`` of ``libg4b_attn.so``
+(hand-written HIP for gfx950); there is no other code path.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+from .. import _native
+from . import utils as U
+
+# g4b/kernels/fa2.py:14-19
+STAGE_FULL = 1
+STAGE_ON_BAND = 2
+STAGE_CAUSAL = STAGE_FULL | STAGE_ON_BAND
+INNER_STAGE_OFF_BAND = 1
+INNER_STAGE_ON_BAND = 2
+INNER_STAGE_FULL = 3
+# g4b/kernels/fa2.py:29-31 -- per-slot phase: 0 unallocated (skipped by every launch), 1 prefill, 2 decode
+PHASE_UNALLOCATED = 0
+PHASE_PREFILL = 1
+PHASE_DECODE = 2
+
+MAX_DECODE_ROWS = 16  # (H/G) * Tq up to which a launch takes the split-KV streaming kernel
+
+_private_workspaces: dict = {}
+
+
+def workspace_bytes(B: int, H: int, G: int, Tq: int, D: int, num_workers: int = 0) -> int:
+    """Bytes of scratch a decode-shaped launch needs to split keys over ``num_workers`` waves."""
+    return int(_native.load().g4b_attn_workspace_bytes(B, H, G, Tq, D, num_workers))
+
+
+def _private_workspace(q, nbytes: int):
+    """Per-device scratch owned by this module, created on first use and grown on demand.
+
+    The reference sizes its split buffers once at load (``g4b/models/gemma4e.py:819-821``) and
+    compiles its kernels during warm-up; this allocation likewise happens on the first call with a
+    given shape, i.e. before a graph is recorded.  Callers that must not allocate at all pass
+    ``workspace=`` explicitly.
+    """
+    import torch
+
+    dev = q.device if hasattr(q, "device") else torch.device("cuda", torch.cuda.current_device())
+    key = str(dev)
+    ws = _private_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _private_workspaces[key] = ws
+    return ws
+
+
+def flash_attention(
+    q,
+    k_cache,
+    v_cache,
+    o,
+    time_dim_sizes,
+    user_phase,
+    ctx_window_size: int,
+    phase: int,
+    partial_o=None,
+    partial_l=None,
+    partial_m=None,
+    *,
+    use_grouped_query_tile: bool = True,
+    warp_specialize: bool = False,
+    is_hopper: bool = False,
+    use_fp32_dot: bool = False,
+    stage: int = STAGE_CAUSAL,
+    scale: float = 1.0,
+    query_window: int | None = None,
+    window_sizes=None,
+    workspace=None,
+    num_workers: int = 0,
+    stream=None,
+):
+    """``o[b, h, i] = softmax(scale * q[b, h, i] . K_b^T + mask) V_b`` for every in-phase slot ``b``.
+
+    Positional arguments and the first five keywords are the reference's (``fa2.py:634-652``):
+
+    * ``q``, ``o``: ``[B, H, Tq, D]`` (strided views allowed, unit stride in ``D``);
+      ``k_cache``, ``v_cache``: ``[B, G, KV_CTX, D]`` rings; ``time_dim_sizes``: ``[B]`` int32;
+      ``user_phase``: ``[B]`` uint8 -- slots with ``user_phase[b] != phase`` are skipped and their
+      rows of ``o`` stay untouched.
+    * ``partial_o/l/m``: the reference's split-KV scratch.  All three or none
+      (``ValueError`` otherwise, ``fa2.py:656-657``).  Passing them allows a decode launch to
+      split keys across workgroups, as in the reference; the partials themselves live in a
+      private workspace (or ``workspace=``) with this library's own layout, and the contents of
+      ``partial_*`` are left unspecified.
+    * ``use_grouped_query_tile``, ``warp_specialize``, ``is_hopper``, ``use_fp32_dot``: tuning
+      knobs of the Triton kernel; accepted and ignored (the GQA group is always packed and the
+      products always run on fp16/bf16 MFMA with fp32 accumulation).
+    * ``stage``: ``STAGE_CAUSAL`` or ``STAGE_FULL``.
+
+    Keyword-only extensions, with defaults that reproduce the reference:
+
+    * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
+      ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
+      ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
+      used for split partials instead of the private one); ``num_workers``; ``stream``.
+
+    Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
+    ignore (``g4b/models/gemma4e.py:593-607``).
+    """
+    assert isinstance(phase, int)  # fa2.py:653
+    if (partial_o is None) != (partial_l is None) or (partial_o is None) != (partial_m is None):
+        raise ValueError("partial_o, partial_l, and partial_m must be provided together")
+
+    U.require_tensor(q, "q", 4)
+    U.require_tensor(o, "o", 4)
+    U.require_tensor(k_cache, "k_cache", 4)
+    U.require_tensor(v_cache, "v_cache", 4)
+    U.require_tensor(time_dim_sizes, "time_dim_sizes", 1)
+    U.require_tensor(user_phase, "user_phase", 1)
+    B, H, Tq, D = U.shape_of(q)
+    Bk, G, KV_CTX, Dk = U.shape_of(k_cache)
+    # the reference's static asserts (fa2.py:289-320)
+    if U.shape_of(o) != [B, H, Tq, D]:
+        raise ValueError(f"o shape {tuple(o.shape)} must equal q shape {tuple(q.shape)}")
+    if U.shape_of(v_cache) != [Bk, G, KV_CTX, Dk]:
+        raise ValueError("k_cache and v_cache must have the same shape")
+    if Bk != B or Dk != D:
+        raise ValueError("q and the caches must agree in batch size and head dim")
+    if U.shape_of(time_dim_sizes) != [B] or U.shape_of(user_phase) != [B]:
+        raise ValueError("time_dim_sizes and user_phase must have shape [B]")
+    if G == 0 or H % G:
+        raise ValueError("number of query heads must be a multiple of the number of kv heads")
+    U.int_itemsize(time_dim_sizes, "time_dim_sizes", {"int32"})
+    U.int_itemsize(user_phase, "user_phase", {"uint8"})
+    ks, vs = U.strides_of(k_cache), U.strides_of(v_cache)
+    for name, s in (("k_cache", ks), ("v_cache", vs)):
+        if s[3] != 1 or s[2] != D or s[1] != KV_CTX * D:  # fa2.py:315-320
+            raise ValueError(f"{name} must be contiguous inside a slot")
+    kv_dt = U.float_dtype_code(k_cache, "k_cache")
+    if U.float_dtype_code(v_cache, "v_cache") != kv_dt:
+        raise ValueError("k_cache and v_cache must have the same dtype")
+    max_kv_splits = 1
+    if partial_o is not None:
+        max_kv_splits = min(int(partial_o.shape[0]), int(partial_l.shape[0]), int(partial_m.shape[0]))  # fa2.py:658
+
+    lib = _native.load()
+    a = _native.AttnArgs()
+    a.q, a.k_cache, a.v_cache, a.o = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr()
+    a.time_dim_sizes, a.user_phase = time_dim_sizes.data_ptr(), user_phase.data_ptr()
+    a.q_stride = (C.c_int64 * 4)(*U.strides_of(q))
+    a.o_stride = (C.c_int64 * 4)(*U.strides_of(o))
+    a.k_stride_b, a.v_stride_b = ks[0], vs[0]
+    a.time_dim_sizes_stride = U.strides_of(time_dim_sizes)[0]
+    a.user_phase_stride = U.strides_of(user_phase)[0]
+    if window_sizes is not None:
+        U.require_tensor(window_sizes, "window_sizes", 1)
+        U.int_itemsize(window_sizes, "window_sizes", {"int32"})
+        if U.shape_of(window_sizes) != [B]:
+            raise ValueError("window_sizes must have shape [B]")
+        a.window_sizes = window_sizes.data_ptr()
+        a.window_sizes_stride = U.strides_of(window_sizes)[0]
+    a.q_dtype = U.float_dtype_code(q, "q")
+    a.o_dtype = U.float_dtype_code(o, "o")
+    a.kv_dtype = kv_dt
+    a.B, a.H, a.G, a.Tq, a.D, a.KV_CTX = B, H, G, Tq, D, KV_CTX
+    a.ctx_window_size = int(ctx_window_size)
+    a.phase = phase
+    a.stage = int(stage)
+    a.query_window = 0 if query_window is None else int(query_window)
+    if query_window is not None and a.query_window < 1:
+        raise ValueError("query_window must be a positive int or None")
+    a.num_workers = int(num_workers)
+    a.scale = float(scale)
+
+    ws = workspace
+    if ws is None and max_kv_splits > 1 and (H // G) * Tq <= MAX_DECODE_ROWS:
+        ws = _private_workspace(q, workspace_bytes(B, H, G, Tq, D, num_workers))
+    if ws is not None:
+        a.workspace = ws.data_ptr()
+        a.workspace_bytes = int(ws.numel()) * int(ws.element_size()) if hasattr(ws, "numel") else int(ws.nbytes)
+
+    _native.check(lib.g4b_attn_forward(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    return None, None

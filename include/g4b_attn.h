@@ -1,0 +1,169 @@
+/*
+ * g4b_attn.h -- C ABI of libg4b_attn.so: the attention hot path of the g4b inference engine
+ * (flash attention over the per-slot ring KV cache, KV append, decode-state advance) as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - Every pointer is a device pointer owned by the caller; the library never allocates,
+ *     frees or synchronises.  Work is enqueued on `stream` (a hipStream_t passed as void*;
+ *     NULL = the default stream) and is legal inside stream capture.
+ *   - Strides are in ELEMENTS, as in the reference's launch adapter (g4b/kernels/utils.py:87-127).
+ *   - Entry points return G4B_OK (0) or a negative g4b_status.  Arguments are validated on the
+ *     host before anything is launched; g4b_last_error() returns a thread-local message for the
+ *     last failure.
+ *   - dtype codes: G4B_DT_F16, G4B_DT_BF16, G4B_DT_F32.
+ */
+#ifndef G4B_ATTN_H
+#define G4B_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define G4B_ATTN_ABI_VERSION 1
+
+enum g4b_status {
+    G4B_OK = 0,
+    G4B_ERR_INVALID_ARGUMENT = -1, /* shape / stride / dtype / value check failed (reference: tl.static_assert) */
+    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim 512, STAGE_ON_BAND alone) */
+    G4B_ERR_WORKSPACE = -3,        /* workspace missing or too small for the requested split-KV launch */
+    G4B_ERR_LAUNCH = -4            /* the HIP runtime refused the launch (no device, bad stream, ...) */
+};
+
+enum g4b_dtype { G4B_DT_F16 = 0, G4B_DT_BF16 = 1, G4B_DT_F32 = 2 };
+
+/* g4b/kernels/fa2.py:14-16 */
+enum g4b_stage { G4B_STAGE_FULL = 1, G4B_STAGE_ON_BAND = 2, G4B_STAGE_CAUSAL = 3 };
+/* g4b/kernels/fa2.py:29-31 */
+enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DECODE = 2 };
+
+/*
+ * g4b_attn_forward replaces flash_attention() = _attn_kernel + _reduce_split_kv_kernel
+ * (g4b/kernels/fa2.py:634-715, 256-480, 546-631).
+ *
+ *   q, o          [B, H, Tq, D], any strides with last stride 1 (the engine passes permuted views
+ *                 of [B, t, H, D] scratchpads, g4b/models/gemma4e.py:1031-1033); f16 / bf16 / f32.
+ *   k_cache,      [B, G, KV_CTX, D], contiguous inside a slot (fa2.py:315-320), slot stride
+ *   v_cache       k_stride_b / v_stride_b; f16 or bf16.
+ *   time_dim_sizes[B] int32: tokens in the slot after this step (fa2.py:52).
+ *   user_phase    [B] uint8: slots whose value differs from `phase` are skipped and their rows of
+ *                 `o` are left untouched (fa2.py:332-335).
+ *   ctx_window_size  W <= KV_CTX: the launch sees the last min(tds, W) keys; logical key j is ring
+ *                 row (max(tds - W, 0) + j) % KV_CTX; query i is aligned with logical key
+ *                 min(tds, W) - Tq + i (fa2.py:53-56,75).
+ *   stage         G4B_STAGE_CAUSAL (default of the reference) or G4B_STAGE_FULL.
+ *   scale         softmax scale; the reference computes with 1.0 (fa2.py:89).
+ *   query_window  0 = anchored window, the reference kernel's semantics.  > 0 additionally hides
+ *                 keys with q_pos - k_pos >= query_window, the per-query sliding window of the CPU
+ *                 reference's one-shot prefill (scripts/reference_impl.py:440-441).
+ *   window_sizes  optional [B] int32 per-slot override of ctx_window_size (extension; NULL = none).
+ *   workspace     device scratch for split-KV partials, >= g4b_attn_workspace_bytes(...) bytes, or
+ *                 NULL: then a decode-shaped launch (R*Tq <= 16) uses one wave per (slot, kv head).
+ *                 Contents are unspecified after the call (like partial_o/l/m, fa2.py:643-645).
+ *   num_workers   0 = library default; otherwise the number of waves the decode key tiles are
+ *                 dealt to (must not exceed the value the workspace was sized for).
+ *
+ * Rows whose visible key set is empty (time_dim_sizes[b] == 0 on an in-phase slot) are written
+ * as zeros; the reference leaves 0/0 there and its caller ignores them (g4b/scheduler.py:142-148).
+ */
+typedef struct g4b_attn_args {
+    const void* q;
+    const void* k_cache;
+    const void* v_cache;
+    void* o;
+    const int32_t* time_dim_sizes;
+    const uint8_t* user_phase;
+    const int32_t* window_sizes;
+    void* workspace;
+    uint64_t workspace_bytes;
+    int64_t q_stride[4];
+    int64_t o_stride[4];
+    int64_t k_stride_b;
+    int64_t v_stride_b;
+    int64_t time_dim_sizes_stride;
+    int64_t user_phase_stride;
+    int64_t window_sizes_stride;
+    int32_t q_dtype;
+    int32_t o_dtype;
+    int32_t kv_dtype;
+    int32_t B, H, G, Tq, D, KV_CTX;
+    int32_t ctx_window_size;
+    int32_t phase;
+    int32_t stage;
+    int32_t query_window;
+    int32_t num_workers;
+    float scale;
+} g4b_attn_args;
+
+int g4b_attn_forward(const g4b_attn_args* args, void* stream);
+
+/* Bytes of workspace that let g4b_attn_forward split the keys of a decode-shaped launch
+ * (R*Tq <= 16) over `num_workers` waves (0 = library default).  Returns 0 when the shape never
+ * uses a workspace (prefill-shaped launches). */
+uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers);
+
+/* The library default for num_workers on the current build (a multiple of the CU count). */
+int32_t g4b_attn_default_workers(void);
+
+/*
+ * g4b_kv_append replaces add_kv_to_cache() (g4b/kernels/add_kv_to_cache.py:84-186):
+ *   cache[b, g, (t + cache_offsets[b]) % T, :] = x[b, g, t, :] * (x_rsos ? rsqrt(x_rsos[b,g,t] / D + eps) : 1)
+ * for slots with user_phase[b] == phase (all slots when user_phase is NULL).
+ *   x [B,G,t,D] strided (last stride 1), f16/bf16/f32; cache [B,G,T,D] contiguous inside a slot,
+ *   f16/bf16/f32; cache_offsets [B] int32 or int64; x_rsos [B,G,t] f32 strided or NULL; t <= T.
+ */
+typedef struct g4b_kv_append_args {
+    const void* x;
+    void* cache;
+    const void* cache_offsets;
+    const float* x_rsos;
+    const uint8_t* user_phase;
+    int64_t x_stride[4];
+    int64_t x_rsos_stride[3];
+    int64_t cache_stride_b;
+    int64_t cache_offsets_stride;
+    int64_t user_phase_stride;
+    int32_t x_dtype;
+    int32_t cache_dtype;
+    int32_t cache_offsets_is_int64;
+    int32_t B, G, t, T, D;
+    int32_t phase;
+    float rmsnorm_eps;
+} g4b_kv_append_args;
+
+int g4b_kv_append(const g4b_kv_append_args* args, void* stream);
+
+/*
+ * g4b_advance_decode_state replaces advance_decode_state()
+ * (g4b/kernels/advance_decode_state.py:32-80): for slots with user_phase[b] == 2,
+ *   input_token_ids[0, b] = out_token_ids[b, 0]; cache_offsets[b] += 1; time_dim_sizes[b] += 1.
+ */
+typedef struct g4b_advance_args {
+    int32_t* input_token_ids;
+    const int32_t* out_token_ids;
+    int32_t* cache_offsets;
+    int32_t* time_dim_sizes;
+    const uint8_t* user_phase;
+    int64_t input_token_ids_stride1;
+    int64_t out_token_ids_stride0;
+    int64_t cache_offsets_stride;
+    int64_t time_dim_sizes_stride;
+    int64_t user_phase_stride;
+    int32_t B;
+} g4b_advance_args;
+
+int g4b_advance_decode_state(const g4b_advance_args* args, void* stream);
+
+/* Message of the calling thread's last failed call ("" if none). */
+const char* g4b_last_error(void);
+
+/* G4B_ATTN_ABI_VERSION the library was built with. */
+int32_t g4b_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* G4B_ATTN_H */

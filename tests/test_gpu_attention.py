@@ -1,0 +1,242 @@
+"""GPU parity of flash_attention (through the C ABI) against the fp64 oracle.
+
+Shapes follow the reference's compare script (tests/compare_scripts/test_fa2.py:51-79), scaled so
+the CPU oracle finishes in seconds: 7 decode shapes (window 1024..., head dim 128/256, GQA 4:1 and
+8:1), prefill chunks on a long context, one-shot causal prefill, one non-causal; half the slots at
+tds = W, half at tds = W + 17 so the ring wraps (:286-290).  Every variant the script compares
+(no split buffers / split buffers) is compared here as well, with assertions.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ATOL_BF16, RTOL_BF16, assert_close, i32, ix, make_case, oracle, partials, u8
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fa(gpu_device):
+    from g4b_amd.kernels import fa2
+
+    return fa2
+
+
+DECODE_CASES = [
+    # name, B, H, G, D, W
+    ("decode_small_w1024", 4, 8, 2, 128, 1024),
+    ("decode_gemma_w4096", 8, 16, 4, 256, 4096),
+    ("decode_gemma_w8192", 4, 16, 4, 256, 8192),
+    ("decode_gemma_w16384", 2, 16, 4, 256, 16384),
+    ("decode_biggroup_w4096", 4, 32, 4, 256, 4096),
+    ("decode_mha_w512", 3, 4, 4, 128, 512),
+    ("decode_group16_w2048", 2, 16, 1, 256, 2048),
+]
+
+
+@pytest.mark.parametrize("case", DECODE_CASES, ids=[c[0] for c in DECODE_CASES])
+@pytest.mark.parametrize("scale", [1.0, 1 / 16])
+def test_decode_matches_oracle_split_and_unsplit(fa, case, scale):
+    name, B, H, G, D, W = case
+    print(f"case {name} scale {scale}", flush=True)
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=1)
+    tds = [W if b % 2 == 0 else W + 17 for b in range(B)]
+    phase = [ix.PHASE_DECODE] * B
+    ref = oracle(q, k, v, tds, phase, W, ix.PHASE_DECODE, scale=scale)
+    # no split buffers: one wave per (slot, kv head)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, ix.PHASE_DECODE, scale=scale)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what=f"{name} unsplit")
+    # split buffers given: keys dealt to many waves, partials merged
+    o2 = torch.full_like(o, 777.0)
+    fa.flash_attention(q, k, v, o2, i32(tds), u8(phase), W, ix.PHASE_DECODE, *partials(4, B, H, 1, D), scale=scale)
+    torch.cuda.synchronize()
+    assert_close(o2.float().cpu().numpy(), ref, what=f"{name} split")
+    # split and unsplit agree far inside the tolerance (test_fa2.py:432-433)
+    assert (o2.float() - o.float()).abs().max().item() < 1e-3
+
+
+@pytest.mark.parametrize("num_workers", [1, 3, 64, 777, 4096])
+def test_decode_any_worker_count_gives_the_same_answer(fa, num_workers):
+    B, H, G, D, W = 5, 8, 2, 256, 2048
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=2)
+    tds = [1, 33, 700, 2048, 2048 + 300]
+    phase = [2] * B
+    ref = oracle(q, k, v, tds, phase, W, 2, scale=0.0625)
+    ws = torch.empty(fa.workspace_bytes(B, H, G, 1, D, num_workers), dtype=torch.uint8, device="cuda")
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 2, scale=0.0625, workspace=ws, num_workers=num_workers)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what=f"workers={num_workers}")
+
+
+@pytest.mark.parametrize("Tq,H,G", [(2, 8, 2), (4, 8, 2), (3, 4, 4), (2, 16, 2), (1, 16, 1)])
+def test_small_query_blocks_take_the_streaming_kernel(fa, Tq, H, G):
+    """(H/G)*Tq <= 16 rows: causal offsets between the rows of one block, wrap, both stages."""
+    B, D, kv_ctx, W = 3, 256, 200, 150
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=3)
+    tds = [Tq, 150, 150 + 77]
+    phase = [1] * B
+    for stage in (ix.STAGE_CAUSAL, ix.STAGE_FULL):
+        for parts in ((), partials(4, B, H, Tq, D)):
+            o.fill_(777.0)
+            ref = oracle(q, k, v, tds, phase, W, 1, stage=stage, scale=0.0625)
+            fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, *parts, stage=stage, scale=0.0625)
+            torch.cuda.synchronize()
+            assert_close(o.float().cpu().numpy(), ref, what=f"Tq={Tq} stage={stage} split={bool(parts)}")
+
+
+PREFILL_CASES = [
+    # name, B, H, G, Tq, kv_ctx, D, W, stage
+    ("prefill_t128_w4096", 2, 16, 4, 128, 4096, 256, 4096, ix.STAGE_CAUSAL),
+    ("prefill_t256_w4096", 1, 16, 4, 256, 4096, 256, 4096, ix.STAGE_CAUSAL),
+    ("prefill_t256_w1024_d128", 2, 8, 2, 256, 1024, 128, 1024, ix.STAGE_CAUSAL),
+    ("full_t256_w256", 2, 16, 4, 256, 256, 256, 256, ix.STAGE_FULL),
+    ("prefill_ragged_t100", 2, 8, 2, 100, 600, 256, 512, ix.STAGE_CAUSAL),
+    ("prefill_mha_t70", 1, 2, 2, 70, 300, 128, 300, ix.STAGE_CAUSAL),
+    ("prefill_group8_t48", 1, 16, 2, 48, 500, 256, 400, ix.STAGE_CAUSAL),
+]
+
+
+@pytest.mark.parametrize("case", PREFILL_CASES, ids=[c[0] for c in PREFILL_CASES])
+@pytest.mark.parametrize("scale", [1.0, 1 / 16])
+def test_prefill_matches_oracle(fa, case, scale):
+    name, B, H, G, Tq, kv_ctx, D, W, stage = case
+    print(f"case {name} scale {scale}", flush=True)
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=4)
+    tds = [W if b % 2 == 0 else W + 17 for b in range(B)]
+    phase = [1] * B
+    ref = oracle(q, k, v, tds, phase, W, 1, stage=stage, scale=scale)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, stage=stage, scale=scale)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what=name)
+
+
+def test_one_shot_causal_prefill_2048(fa):
+    """BASELINE config 2: batch 1, seq 2048, 8 q heads / 2 kv heads, head dim 256, scale 1/16."""
+    B, H, G, Tq, D = 1, 8, 2, 2048, 256
+    q, k, v, o = make_case(B, H, G, Tq, D, Tq, seed=0)
+    ref = oracle(q, k, v, [Tq], [1], Tq, 1, scale=1 / 16)
+    fa.flash_attention(q, k, v, o, i32([Tq]), u8([1]), Tq, 1, scale=1 / 16)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what="config 2")
+
+
+@pytest.mark.parametrize("qw", [1, 37, 64, 512, 5000])
+def test_per_query_sliding_window(fa, qw):
+    """One-shot prefill longer than the window: key visible iff 0 <= q_pos - k_pos < query_window."""
+    B, H, G, Tq, D = 1, 8, 2, 1024, 256
+    q, k, v, o = make_case(B, H, G, Tq, D, Tq, seed=5)
+    ref = oracle(q, k, v, [Tq], [1], Tq, 1, scale=1 / 16, query_window=qw)
+    fa.flash_attention(q, k, v, o, i32([Tq]), u8([1]), Tq, 1, scale=1 / 16, query_window=qw)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what=f"query_window={qw}")
+
+
+def test_chunk_on_long_context_with_wrap(fa):
+    """A 512-token chunk appended to an existing context in a ring of W + t - 1 rows (gemma4e.py:703-705)."""
+    B, H, G, t, D, W = 2, 8, 2, 512, 256, 2048
+    kv_ctx = W + t - 1
+    q, k, v, o = make_case(B, H, G, t, D, kv_ctx, seed=6)
+    tds = [1500 + t, 9000 + t]  # second slot: window full, ring wrapped several times
+    ref = oracle(q, k, v, tds, [1, 1], W, 1, scale=1 / 16)
+    fa.flash_attention(q, k, v, o, i32(tds), u8([1, 1]), W, 1, scale=1 / 16)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what="chunk on context")
+
+
+def test_phase_skip_leaves_rows_untouched_and_empty_slots_are_zero(fa):
+    B, H, G, D, W = 6, 8, 2, 256, 256
+    for Tq in (1, 64):
+        q, k, v, o = make_case(B, H, G, Tq, D, W, seed=7)
+        phase = [1, 2, 0, 1, 2, 1]
+        tds = [max(Tq, 100), 100, 100, 0, 0, 256 + 40]
+        for launch_phase in (1, 2):
+            o.fill_(777.0)
+            parts = partials(4, B, H, Tq, D) if Tq == 1 else ()
+            fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, launch_phase, *parts, scale=0.0625)
+            torch.cuda.synchronize()
+            got = o.float().cpu().numpy()
+            ref = oracle(q, k, v, tds, phase, W, launch_phase, scale=0.0625)
+            for b in range(B):
+                if phase[b] != launch_phase:
+                    assert (got[b] == 777.0).all(), f"slot {b} of an off-phase launch was written"
+                elif tds[b] == 0:
+                    assert (got[b] == 0).all(), "in-phase slot without keys must be zeros"
+                else:
+                    assert_close(got[b], ref[b], what=f"Tq={Tq} slot {b}")
+
+
+@pytest.mark.parametrize("Tq", [1, 96])
+def test_engine_layout_fp32_strided_views(fa, Tq):
+    """q and o as the engine passes them: fp32, permuted views of [B, t, H, D] scratchpads (gemma4e.py:1031-1033)."""
+    B, H, G, D, W = 3, 8, 2, 256, 700
+    q, k, v, o = make_case(B, H, G, Tq, D, W, seed=8, q_dtype=torch.float32, engine_layout=True)
+    assert not q.is_contiguous() or Tq == 1
+    tds = [W, W + 17, max(Tq, 5)]
+    phase_id = 2 if Tq == 1 else 1
+    # the MFMA path rounds q to fp16 first; compare against the oracle on the rounded values
+    ref = oracle(q.half(), k, v, tds, [phase_id] * B, W, phase_id, scale=0.0625)
+    parts = partials(16, B, H, Tq, D) if Tq == 1 else ()
+    fa.flash_attention(q, k, v, o, i32(tds), u8([phase_id] * B), W, phase_id, *parts, scale=0.0625, use_fp32_dot=True)
+    torch.cuda.synchronize()
+    assert o.dtype == torch.float32
+    assert_close(o.cpu().numpy(), ref, what="engine layout")
+
+
+@pytest.mark.parametrize("Tq", [1, 160])
+def test_bf16_cache(fa, Tq):
+    B, H, G, D, W = 2, 8, 2, 256, 1024
+    q, k, v, o = make_case(B, H, G, Tq, D, W, seed=9, dtype=torch.bfloat16)
+    tds = [W, W + 17]
+    phase_id = 2 if Tq == 1 else 1
+    ref = oracle(q, k, v, tds, [phase_id] * B, W, phase_id, scale=0.0625)
+    parts = partials(4, B, H, Tq, D) if Tq == 1 else ()
+    fa.flash_attention(q, k, v, o, i32(tds), u8([phase_id] * B), W, phase_id, *parts, scale=0.0625)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, atol=ATOL_BF16, rtol=RTOL_BF16, what="bf16")
+
+
+@pytest.mark.parametrize("Tq", [1, 4, 40])
+def test_visible_set_is_bit_exact(fa, Tq):
+    """K = 0 makes the weights uniform; V row r = e_(r mod D) turns the output into the indicator of the
+    ring rows that were read divided by their count, so the visible set is read back exactly."""
+    B, H, G, D = 4, 8, 2, 256
+    kv_ctx, W = 251, 200  # W <= KV_CTX <= D so that every ring row has its own output column
+    q = torch.randn(B, H, Tq, D, device="cuda").half()
+    k = torch.zeros(B, G, kv_ctx, D, device="cuda", dtype=torch.float16)
+    v = torch.zeros(B, G, kv_ctx, D, device="cuda", dtype=torch.float16)
+    v[:, :, torch.arange(kv_ctx), torch.arange(kv_ctx)] = 1.0
+    tds = [Tq, 57 + Tq, 200, 200 + 123]
+    phase_id = 2 if Tq == 1 else 1
+    for qw in (None, 7):
+        o = torch.zeros(B, H, Tq, D, device="cuda", dtype=torch.float32)
+        parts = partials(4, B, H, Tq, D) if Tq * 4 <= 16 else ()
+        fa.flash_attention(q, k, v, o, i32(tds), u8([phase_id] * B), W, phase_id, *parts, query_window=qw)
+        torch.cuda.synchronize()
+        got = o.cpu().numpy()
+        for b in range(B):
+            for i in range(Tq):
+                lo, hi = ix.visible_range(i, tds[b], W, Tq, ix.STAGE_CAUSAL, qw)
+                rows = sorted(ix.ring_row(tds[b], W, kv_ctx, j) for j in range(lo, hi))
+                for h in range(H):
+                    read = np.nonzero(got[b, h, i])[0].tolist()
+                    assert read == rows, (Tq, qw, b, h, i)
+                    np.testing.assert_allclose(got[b, h, i, rows], 1.0 / len(rows), rtol=2e-3)
+
+
+def test_argument_errors_follow_the_reference(fa):
+    B, H, G, D, W = 2, 8, 2, 256, 64
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=10)
+    tds, ph = i32([10, 20]), u8([2, 2])
+    po, pl, pm = partials(4, B, H, 1, D)
+    with pytest.raises(ValueError):  # fa2.py:656-657
+        fa.flash_attention(q, k, v, o, tds, ph, W, 2, po, None, pm)
+    with pytest.raises(AssertionError):  # fa2.py:653
+        fa.flash_attention(q, k, v, o, tds, ph, W, 2.0)
+    with pytest.raises(ValueError):  # fa2.py:298 ctx_window_size <= KV_CTX
+        fa.flash_attention(q, k, v, o, tds, ph, W + 1, 2)
+    with pytest.raises(ValueError):  # fa2.py:293
+        fa.flash_attention(q, k, v, o[:, :4], tds, ph, W, 2)
+    with pytest.raises(NotImplementedError):
+        fa.flash_attention(q, k, v, o, tds, ph, W, 2, stage=fa.STAGE_ON_BAND)

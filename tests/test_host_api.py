@@ -1,0 +1,176 @@
+"""CPU-side checks of the C ABI and the Python boundary (no GPU, no compute calls)."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+@pytest.fixture(scope="module")
+def native():
+    from g4b_amd import _native
+
+    if not _native.LIB_PATH.exists():
+        from g4b_amd.build import build
+
+        build()
+    _native.load()
+    return _native
+
+
+def test_library_exports_every_declared_symbol(native):
+    header = (ROOT / "include" / "g4b_attn.h").read_text()
+    declared = set(re.findall(r"\b(g4b_[a-z_]+)\s*\(", header))
+    assert declared == set(native.EXPORTS), declared ^ set(native.EXPORTS)
+    lib = ctypes.CDLL(str(native.LIB_PATH))
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.g4b_abi_version() == native.ABI_VERSION
+
+
+def test_struct_layouts_match_the_header(native):
+    """Field order and C types of the ctypes mirrors follow the header's structs."""
+    header = (ROOT / "include" / "g4b_attn.h").read_text()
+    ctype_of = {
+        "void*": ctypes.c_void_p,
+        "int32_t*": ctypes.c_void_p,
+        "uint8_t*": ctypes.c_void_p,
+        "float*": ctypes.c_void_p,
+        "uint64_t": ctypes.c_uint64,
+        "int64_t": ctypes.c_int64,
+        "int32_t": ctypes.c_int32,
+        "float": ctypes.c_float,
+    }
+    for cname, mirror in (
+        ("g4b_attn_args", native.AttnArgs),
+        ("g4b_kv_append_args", native.KvAppendArgs),
+        ("g4b_advance_args", native.AdvanceArgs),
+    ):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), header, re.S).group(1)
+        fields = []
+        for line in body.splitlines():
+            line = line.split("/*")[0].strip().rstrip(";")
+            if not line:
+                continue
+            m = re.match(r"(?:const\s+)?([a-z0-9_]+\s*\*?)\s*(.*)", line)
+            ctype = m.group(1).replace(" ", "")
+            for decl in m.group(2).split(","):
+                decl = decl.strip()
+                arr = re.match(r"(\w+)\[(\d+)\]", decl)
+                if arr:
+                    fields.append((arr.group(1), ctype_of[ctype] * int(arr.group(2))))
+                else:
+                    fields.append((decl, ctype_of[ctype]))
+        got = [(n, t) for n, t in mirror._fields_]
+        assert [n for n, _ in got] == [n for n, _ in fields], cname
+        for (n, t), (_, t2) in zip(got, fields):
+            assert ctypes.sizeof(t) == ctypes.sizeof(t2), (cname, n)
+
+
+def test_workspace_size_formula(native):
+    lib = native.load()
+    nw = lib.g4b_attn_default_workers()
+    assert nw > 0
+    # (workers + B*G) partial slots of rows x (D + 2) floats
+    assert lib.g4b_attn_workspace_bytes(64, 8, 2, 1, 256, 0) == (nw + 128) * 4 * 258 * 4
+    assert lib.g4b_attn_workspace_bytes(3, 8, 2, 2, 128, 10) == (10 + 6) * 8 * 130 * 4
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 512, 256, 0) == 0  # prefill-shaped: no workspace
+
+
+def _decode_args():
+    q = torch.zeros(2, 8, 1, 256, dtype=torch.float16)
+    k = torch.zeros(2, 2, 64, 256, dtype=torch.float16)
+    return q, k, k.clone(), q.clone(), torch.zeros(2, dtype=torch.int32), torch.zeros(2, dtype=torch.uint8)
+
+
+def test_python_boundary_validates_like_the_reference(native):
+    from g4b_amd.kernels.fa2 import PHASE_DECODE, STAGE_CAUSAL, STAGE_FULL, STAGE_ON_BAND, flash_attention
+
+    assert (STAGE_FULL, STAGE_ON_BAND, STAGE_CAUSAL) == (1, 2, 3)  # fa2.py:14-16
+    q, k, v, o, tds, ph = _decode_args()
+    with pytest.raises(ValueError, match="provided together"):  # fa2.py:656-657
+        flash_attention(q, k, v, o, tds, ph, 64, PHASE_DECODE, torch.zeros(4, 2, 8, 1, 256))
+    with pytest.raises(AssertionError):  # fa2.py:653
+        flash_attention(q, k, v, o, tds, ph, 64, "decode")
+    with pytest.raises(ValueError, match="ctx_window_size"):  # fa2.py:298
+        flash_attention(q, k, v, o, tds, ph, 65, PHASE_DECODE)
+    with pytest.raises(ValueError):  # fa2.py:296
+        flash_attention(q[:, :7], k, v, o[:, :7], tds, ph, 64, PHASE_DECODE)
+    with pytest.raises(ValueError, match="contiguous"):  # fa2.py:315-320
+        flash_attention(q, k[:, :, ::2], v[:, :, ::2], o, tds, ph, 32, PHASE_DECODE)
+    with pytest.raises(ValueError):
+        flash_attention(q, k, v, o, tds.long(), ph, 64, PHASE_DECODE)
+    with pytest.raises(NotImplementedError):
+        flash_attention(q, k, v, o, tds, ph, 64, PHASE_DECODE, stage=STAGE_ON_BAND)
+    q5, k5 = torch.zeros(2, 8, 1, 512, dtype=torch.float16), torch.zeros(2, 2, 64, 512, dtype=torch.float16)
+    with pytest.raises(NotImplementedError, match="head_dim"):
+        flash_attention(q5, k5, k5, q5.clone(), tds, ph, 64, PHASE_DECODE)
+
+
+def test_c_abi_rejects_bad_arguments_before_launching(native):
+    lib = native.load()
+    assert lib.g4b_attn_forward(None, None) == native.G4B_ERR_INVALID_ARGUMENT
+    assert "NULL" in native.last_error()
+    a = native.AttnArgs()
+    assert lib.g4b_attn_forward(ctypes.byref(a), None) == native.G4B_ERR_INVALID_ARGUMENT
+    k = native.KvAppendArgs()
+    assert lib.g4b_kv_append(ctypes.byref(k), None) == native.G4B_ERR_INVALID_ARGUMENT
+    adv = native.AdvanceArgs()
+    assert lib.g4b_advance_decode_state(ctypes.byref(adv), None) == native.G4B_ERR_INVALID_ARGUMENT
+    # workspace too small is reported, not launched
+    q, kk, v, o, tds, ph = _decode_args()
+    from g4b_amd.kernels.fa2 import flash_attention
+
+    with pytest.raises(ValueError, match="workspace"):
+        flash_attention(q, kk, v, o, tds, ph, 64, 2, workspace=torch.zeros(64, dtype=torch.uint8))
+
+
+def test_kv_append_and_advance_validation(native):
+    from g4b_amd.kernels.add_kv_to_cache import add_kv_to_cache
+    from g4b_amd.kernels.advance_decode_state import advance_decode_state
+
+    x = torch.zeros(2, 4, 7, 256)
+    cache = torch.zeros(2, 4, 17, 256, dtype=torch.float16)
+    offs = torch.tensor([15, 3])
+    with pytest.raises(AssertionError):  # add_kv_to_cache.py:171
+        add_kv_to_cache(x, cache, offs, 1e-6, phase=1.0)
+    with pytest.raises(ValueError):  # add_kv_to_cache.py:119
+        add_kv_to_cache(torch.zeros(2, 4, 18, 256), cache, offs, 1e-6)
+    with pytest.raises(ValueError):  # add_kv_to_cache.py:105-107
+        add_kv_to_cache(x, cache[:, :2], offs, 1e-6)
+    with pytest.raises(ValueError):
+        add_kv_to_cache(x, cache, offs, 1e-6, x_rsos=torch.zeros(2, 4, 6))
+    with pytest.raises(ValueError):  # advance_decode_state.py:45-50
+        advance_decode_state(
+            torch.zeros(1, 3, dtype=torch.int32),
+            torch.zeros(4, 1, dtype=torch.int32),
+            torch.zeros(3, dtype=torch.int32),
+            torch.zeros(3, dtype=torch.int32),
+            torch.zeros(3, dtype=torch.uint8),
+        )
+
+
+def test_tensor_protocol_accepts_g4b_style_tensors(native):
+    """Objects with shape / stride sequence / dtype.name / data_ptr() (g4b/tensor.py:71-80) are accepted."""
+    from g4b_amd.kernels import utils as U
+
+    class DT:
+        def __init__(self, name):
+            self.name = name
+
+    class T:
+        def __init__(self, t, name):
+            self._t, self.shape, self.stride, self.dtype = t, list(t.shape), list(t.stride()), DT(name)
+
+        def data_ptr(self):
+            return self._t.data_ptr()
+
+    t = torch.zeros(2, 3, 4, 8, dtype=torch.float16).permute(0, 2, 1, 3)
+    w = T(t, "float16")
+    assert U.strides_of(w) == list(t.stride()) == U.strides_of(t)
+    assert U.float_dtype_code(w, "w") == U.float_dtype_code(t, "t") == native.DT_F16
+    assert U.dtype_name(torch.zeros(1, dtype=torch.int32)) == "int32"

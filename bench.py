@@ -1,0 +1,431 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu-baseline]
+
+A "step" is one pass of the hot path over one batch of synthetic input: one ``flash_attention``
+call (all of its kernels) on inputs that already sit in HBM.  The default workload is the batched
+decode configuration of the metric (64 sequences, KV lengths U{128..32768}, half of them with a
+512-token sliding window); ``value`` is its algorithmic KV bytes per second.  The other synthetic
+configurations (single-sequence decode, causal prefill 2048 / 8192, sliding-window prefill 8192, the
+mixed chunked-prefill step) are timed as well and reported under ``extra`` unless ``--no-extra``.
+
+One JSON line is printed at the end.  ``roofline`` describes the dominant kernel of the primary
+workload: algorithmic bytes (or flops) per launch divided by that kernel's average duration,
+measured here with HIP events on the launch stream.  ``cpu_baseline`` is the CPU restatement of the
+reference attention timed on the host cores on a bounded sample of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "decode attn GB/s (% HBM peak); prefill attn TFLOP/s (% fp16 MFMA peak)"
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+H, G, D = 8, 2, 256
+SCALE = 1.0 / 16.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+# --------------------------------------------------------------------------- workloads
+class Workload:
+    """Device tensors plus the closures that launch the hot path on them."""
+
+    name = ""
+    bound = "hbm"
+
+    def launch(self, i: int = 0, kernel_mask: int = 0):
+        raise NotImplementedError
+
+    def cpu_sample(self):
+        """-> (seconds, units_done, description) for the CPU baseline on a bounded sample."""
+        raise NotImplementedError
+
+
+def _randn_f16(shape, seed, device):
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    return torch.randn(shape, generator=g, device=device, dtype=torch.float16)
+
+
+class BatchedDecode(Workload):
+    """64 sequences x 1 query token against per-sequence ring caches; lengths U{lo..hi}; even slots SWA-512."""
+
+    bound = "hbm"
+
+    def __init__(self, device, B=64, kv_ctx=32768, len_lo=128, len_hi=32768, swa_every=2, seed=0, name="decode_batched_b64"):
+        import numpy as np
+        import torch
+
+        from g4b_amd.kernels import fa2
+
+        self.name = name
+        self.fa2 = fa2
+        self.B, self.kv_ctx = B, kv_ctx
+        rng = np.random.default_rng(seed)
+        self.tds_list = rng.integers(len_lo, len_hi + 1, B).tolist()
+        self.win_list = [512 if (swa_every and b % swa_every == 0) else kv_ctx for b in range(B)]
+        self.n_keys = [min(t, w) for t, w in zip(self.tds_list, self.win_list)]
+        self.q = _randn_f16((B, H, 1, D), seed + 1, device)
+        self.k = _randn_f16((B, G, kv_ctx, D), seed + 2, device)
+        self.v = _randn_f16((B, G, kv_ctx, D), seed + 3, device)
+        self.o = torch.empty_like(self.q)
+        self.tds = torch.tensor(self.tds_list, dtype=torch.int32, device=device)
+        self.win = torch.tensor(self.win_list, dtype=torch.int32, device=device)
+        self.phase = torch.full((B,), fa2.PHASE_DECODE, dtype=torch.uint8, device=device)
+        self.ws = torch.empty(fa2.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device=device)
+        # algorithmic bytes: every visible K and V row once per kv head (2 * G * D * 2 bytes per key)
+        self.bytes = 2 * G * D * 2 * sum(self.n_keys)
+        self.flops = 4 * H * D * sum(self.n_keys)
+        self.units = self.bytes
+
+    def launch(self, i=0, kernel_mask=0):
+        self.fa2.flash_attention(
+            self.q, self.k, self.v, self.o, self.tds, self.phase, self.kv_ctx, self.fa2.PHASE_DECODE,
+            scale=SCALE, window_sizes=self.win, workspace=self.ws, kernel_mask=kernel_mask,
+        )
+
+    def cpu_sample(self):
+        import torch
+
+        from oracle import attention_ref as ar
+
+        slots = list(range(min(self.B, 16)))
+        q, k, v = self.q[slots].cpu(), self.k[slots].cpu(), self.v[slots].cpu()
+        tds = [self.tds_list[b] for b in slots]
+        win = [self.win_list[b] for b in slots]
+        t0 = time.perf_counter()
+        ar.attention_cpu_baseline(q, k, v, tds, [2] * len(slots), self.kv_ctx, 2, scale=SCALE, window_sizes=win)
+        dt = time.perf_counter() - t0
+        done = 2 * G * D * 2 * sum(self.n_keys[b] for b in slots)
+        return dt, done, f"slots 0..{len(slots) - 1} of {self.B} ({done / 1e6:.1f} MB of KV), one pass"
+
+
+class SingleDecode(Workload):
+    """Config 1: one sequence, KV length 2048.  64 distinct caches are rotated so that the 4 MiB do not sit in cache."""
+
+    bound = "hbm"
+
+    def __init__(self, device, n=2048, copies=64, seed=0):
+        import torch
+
+        from g4b_amd.kernels import fa2
+
+        self.name = "decode_single_kv2048"
+        self.fa2 = fa2
+        self.n, self.copies = n, copies
+        self.q = _randn_f16((copies, H, 1, D), seed + 1, device)
+        self.k = _randn_f16((copies, G, n, D), seed + 2, device)
+        self.v = _randn_f16((copies, G, n, D), seed + 3, device)
+        self.o = torch.empty_like(self.q)
+        self.tds = torch.full((1,), n, dtype=torch.int32, device=device)
+        self.phase = torch.full((1,), fa2.PHASE_DECODE, dtype=torch.uint8, device=device)
+        self.ws = torch.empty(fa2.workspace_bytes(1, H, G, 1, D), dtype=torch.uint8, device=device)
+        self.bytes = 2 * G * n * D * 2
+        self.flops = 4 * H * n * D
+        self.units = self.bytes
+
+    def launch(self, i=0, kernel_mask=0):
+        c = i % self.copies
+        self.fa2.flash_attention(
+            self.q[c : c + 1], self.k[c : c + 1], self.v[c : c + 1], self.o[c : c + 1], self.tds, self.phase,
+            self.n, self.fa2.PHASE_DECODE, scale=SCALE, workspace=self.ws, kernel_mask=kernel_mask,
+        )
+
+    def cpu_sample(self):
+        from oracle import attention_ref as ar
+
+        q, k, v = self.q[:1].cpu(), self.k[:1].cpu(), self.v[:1].cpu()
+        reps = 20
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            ar.attention_cpu_baseline(q, k, v, [self.n], [2], self.n, 2, scale=SCALE)
+        dt = time.perf_counter() - t0
+        return dt, reps * self.bytes, f"{reps} passes over one cache"
+
+
+class Prefill(Workload):
+    """One-shot prefill: batch 1, Tq = S tokens, causal; ``query_window`` turns it into the per-query sliding window."""
+
+    bound = "mfma"
+
+    def __init__(self, device, S, query_window=None, seed=0):
+        import torch
+
+        from g4b_amd.kernels import fa2
+
+        self.fa2 = fa2
+        self.S, self.qw = S, query_window
+        self.name = f"prefill_causal_{S}" if query_window is None else f"prefill_swa{query_window}_{S}"
+        self.q = _randn_f16((1, H, S, D), seed + 1, device)
+        self.k = _randn_f16((1, G, S, D), seed + 2, device)
+        self.v = _randn_f16((1, G, S, D), seed + 3, device)
+        self.o = torch.empty_like(self.q)
+        self.tds = torch.full((1,), S, dtype=torch.int32, device=device)
+        self.phase = torch.full((1,), fa2.PHASE_PREFILL, dtype=torch.uint8, device=device)
+        if query_window is None:
+            pairs = S * (S + 1) // 2
+        else:
+            w = query_window
+            pairs = w * (w + 1) // 2 + (S - w) * w
+        self.pairs = pairs
+        self.flops = 4 * H * D * pairs
+        self.bytes = (2 * H * S * D + 2 * G * S * D) * 2
+        self.units = self.flops
+
+    def launch(self, i=0, kernel_mask=0):
+        self.fa2.flash_attention(
+            self.q, self.k, self.v, self.o, self.tds, self.phase, self.S, self.fa2.PHASE_PREFILL,
+            scale=SCALE, query_window=self.qw,
+        )
+
+    def cpu_sample(self):
+        from oracle import attention_ref as ar
+
+        # the last `rows` query rows only (they are the most expensive ones): bounded work, stated in the report
+        rows = min(self.S, 1024)
+        q = self.q[:, :, self.S - rows :].cpu()
+        k, v = self.k.cpu(), self.v.cpu()
+        t0 = time.perf_counter()
+        ar.retrieve_ref_torch(q, k, v, scale=SCALE, query_window=self.qw)
+        dt = time.perf_counter() - t0
+        if self.qw is None:
+            pairs = sum(self.S - rows + i + 1 for i in range(rows))
+        else:
+            pairs = sum(min(self.qw, self.S - rows + i + 1) for i in range(rows))
+        # the dense CPU formulation computes every (row, key) score, masked or not
+        return dt, 4 * H * D * pairs, f"last {rows} query rows against all {self.S} keys (dense scores)"
+
+
+class MixedStep(Workload):
+    """Config 5: 32 decode slots (lengths U{1024..16384}) + one 512-token chunk on a 16384-token context,
+    35 layers alternating sliding-window-512 and global attention; per layer one prefill-phase and one
+    decode-phase launch over the same batch tensors.  The same cache pair is reused by all layers of a kind."""
+
+    bound = "hbm"
+
+    def __init__(self, device, seed=0, layers=35):
+        import numpy as np
+        import torch
+
+        from g4b_amd.kernels import fa2
+
+        self.name = "mixed_step_35_layers"
+        self.fa2 = fa2
+        self.layers = layers
+        B, t, ctx = 33, 512, 16384
+        self.B, self.t = B, t
+        rng = np.random.default_rng(seed)
+        dec_len = rng.integers(1024, 16384 + 1, 32).tolist()
+        self.tds_list = dec_len + [ctx + t]
+        self.T_global, self.T_swa, self.W_swa = 32768 + t - 1, 512 + t - 1, 512
+        self.W_global = 32768
+        self.qp = _randn_f16((B, H, t, D), seed + 1, device)
+        self.qd = _randn_f16((B, H, 1, D), seed + 2, device)
+        self.op, self.od = torch.empty_like(self.qp), torch.empty_like(self.qd)
+        self.kg = _randn_f16((B, G, self.T_global, D), seed + 3, device)
+        self.vg = _randn_f16((B, G, self.T_global, D), seed + 4, device)
+        self.ks = _randn_f16((B, G, self.T_swa, D), seed + 5, device)
+        self.vs = _randn_f16((B, G, self.T_swa, D), seed + 6, device)
+        self.tds = torch.tensor(self.tds_list, dtype=torch.int32, device=device)
+        self.phase = torch.tensor([2] * 32 + [1], dtype=torch.uint8, device=device)
+        self.ws = torch.empty(fa2.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device=device)
+        n_swa, n_glob = (layers + 1) // 2, layers // 2
+        dec_g = 2 * G * D * 2 * sum(min(x, self.W_global) for x in dec_len)
+        dec_s = 2 * G * D * 2 * sum(min(x, self.W_swa) for x in dec_len)
+        pre_g_pairs = t * ctx + t * (t + 1) // 2
+        pre_s_pairs = t * (t + 1) // 2  # anchored window: a chunk of W tokens sees only itself
+        self.bytes = n_glob * dec_g + n_swa * dec_s
+        self.flops = 4 * H * D * (n_glob * pre_g_pairs + n_swa * pre_s_pairs)
+        self.units = self.bytes
+        self.detail = {
+            "decode_bytes_global_layer": dec_g, "decode_bytes_swa_layer": dec_s,
+            "prefill_flops_global_layer": 4 * H * D * pre_g_pairs, "prefill_flops_swa_layer": 4 * H * D * pre_s_pairs,
+        }
+
+    def launch(self, i=0, kernel_mask=0):
+        fa2 = self.fa2
+        for layer in range(self.layers):
+            swa = layer % 2 == 0
+            k, v, W = (self.ks, self.vs, self.W_swa) if swa else (self.kg, self.vg, self.W_global)
+            fa2.flash_attention(self.qp, k, v, self.op, self.tds, self.phase, W, fa2.PHASE_PREFILL, scale=SCALE)
+            fa2.flash_attention(self.qd, k, v, self.od, self.tds, self.phase, W, fa2.PHASE_DECODE, scale=SCALE, workspace=self.ws)
+
+    def cpu_sample(self):
+        raise NotImplementedError
+
+
+WORKLOADS = {
+    "decode_batched": lambda dev: BatchedDecode(dev),
+    "decode_single": lambda dev: SingleDecode(dev),
+    "prefill_causal_2048": lambda dev: Prefill(dev, 2048),
+    "prefill_causal_8192": lambda dev: Prefill(dev, 8192),
+    "prefill_swa_8192": lambda dev: Prefill(dev, 8192, query_window=512),
+    "mixed_step": lambda dev: MixedStep(dev),
+}
+
+
+# --------------------------------------------------------------------------- timing
+def time_steps(wl: Workload, steps: int, warmup: int):
+    """Wall-clock of exactly ``steps`` steps between two device synchronisations -> ms per step."""
+    import torch
+
+    for i in range(warmup):
+        wl.launch(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        wl.launch(warmup + i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def time_kernel_events(wl: Workload, steps: int, kernel_mask: int):
+    """Average GPU duration (ms) of one launch of the selected kernel(s), HIP events on the launch stream."""
+    import torch
+
+    stream = torch.cuda.current_stream()
+    pairs = []
+    for i in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        wl.launch(i, kernel_mask)
+        b.record(stream)
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in pairs)
+    return sum(ts) / len(ts), ts[len(ts) // 2]
+
+
+def measure(wl: Workload, steps: int, warmup: int):
+    ms = time_steps(wl, steps, warmup)
+    kmask = 1 if wl.bound == "hbm" and not isinstance(wl, MixedStep) else 0
+    k_avg, k_med = time_kernel_events(wl, max(steps, 10), kmask)
+    wl.launch(0, 0)  # leave complete results behind after kernel-only launches
+    res = {"ms_per_step": ms, "kernel_ms_avg": k_avg, "kernel_ms_median": k_med}
+    res["GBps"] = wl.bytes / (ms * 1e-3) / 1e9
+    res["TFLOPs"] = wl.flops / (ms * 1e-3) / 1e12
+    if wl.bound == "hbm":
+        ach = wl.bytes / (k_avg * 1e-3) / 1e9
+        res["roofline"] = {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None}
+    else:
+        ach = wl.flops / (k_avg * 1e-3) / 1e12
+        res["roofline"] = {"bound": "mfma", "achieved": round(ach, 1), "peak": FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                           "frac": round(ach / FP16_PEAK_TFLOPS, 4), "traffic": None}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="decode_batched", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extra", action="store_true", help="time the primary workload only")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 1 GiB device-to-device copies (a kernel of known traffic, used to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the attention path shards by slot or kv head with "
+                 "no exchange; nothing here uses a second device). Run with --gpus 1.")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import g4b_amd.kernels  # noqa: F401  raises when libg4b_attn.so is missing
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(dev)
+    log(f"device: {props.name}, {props.multi_processor_count} CUs, {props.total_memory / 2**30:.0f} GiB")
+    log(f"peaks used: HBM {HBM_PEAK_GBPS:.0f} GB/s, fp16 dense MFMA {FP16_PEAK_TFLOPS:.0f} TFLOP/s")
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 29, dtype=torch.float16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        log("copy calibration: 3 copies, each reads 1 GiB and writes 1 GiB")
+        del src, dst
+
+    wl = WORKLOADS[args.workload](dev)
+    res = measure(wl, args.steps, args.warmup)
+    log(f"{wl.name}: {res['ms_per_step']:.4f} ms/step, {res['GBps']:.1f} GB/s, {res['TFLOPs']:.2f} TFLOP/s, "
+        f"kernel {res['kernel_ms_avg']:.4f} ms avg -> {res['roofline']}")
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        try:
+            torch.set_num_threads(os.cpu_count() or 1)
+            secs, done, desc = wl.cpu_sample()
+            unit, val = ("GB/s", done / secs / 1e9) if wl.bound == "hbm" else ("TFLOP/s", done / secs / 1e12)
+            cpu = {"value": round(val, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
+                   "sample": f"{desc}; {secs:.2f} s; torch CPU fp32 restatement of scripts/reference_impl.py:421-443"}
+            log(f"cpu baseline: {cpu}")
+        except NotImplementedError:
+            cpu = None
+
+    extra = {}
+    if not args.no_extra:
+        del wl
+        torch.cuda.empty_cache()
+        for name, make in WORKLOADS.items():
+            if name == args.workload:
+                continue
+            w = make(dev)
+            steps = 3 if name == "mixed_step" else min(args.steps, 20)
+            r = measure(w, steps, min(args.warmup, 3))
+            entry = {"ms_per_step": round(r["ms_per_step"], 4), "GB/s": round(r["GBps"], 1),
+                     "TFLOP/s": round(r["TFLOPs"], 2), "roofline": r["roofline"]}
+            if isinstance(w, MixedStep):
+                entry["detail"] = w.detail
+                entry.pop("roofline")
+            extra[w.name] = entry
+            log(f"{w.name}: {entry}")
+            del w
+            torch.cuda.empty_cache()
+
+    primary_is_hbm = res["roofline"]["bound"] == "hbm"
+    line = {
+        "metric": METRIC,
+        "value": round(res["GBps"] if primary_is_hbm else res["TFLOPs"], 2),
+        "unit": "GB/s" if primary_is_hbm else "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(res["ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "H": H, "G": G, "D": D, "scale": SCALE,
+                   "detail": "fp16 Q/K/V ~ N(0,1) seeded, fp32 softmax accumulation"},
+        "roofline": res["roofline"],
+        "cpu_baseline": cpu,
+        "device": props.name,
+        "extra": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

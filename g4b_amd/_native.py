@@ -49,6 +49,7 @@ class AttnArgs(C.Structure):
         ("stage", C.c_int32),
         ("query_window", C.c_int32),
         ("num_workers", C.c_int32),
+        ("kernel_mask", C.c_int32),
         ("scale", C.c_float),
     ]
 

@@ -110,6 +110,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     p.stage = a->stage;
     p.qwin = a->query_window;
     p.c = a->scale * 1.44269504088896340736f;
+    p.kernel_mask = (a->kernel_mask & 3) ? (a->kernel_mask & 3) : 3;
 
     const int64_t rows = (int64_t)p.R * p.Tq;
     hipError_t e;

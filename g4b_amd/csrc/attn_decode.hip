@@ -359,10 +359,12 @@ __global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
 
 template <int D, int CL, class T>
 static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL((attn_decode_worker<D, CL, T>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64), 0, stream, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G), dim3(256), 0, stream, p);
+    if (p.kernel_mask & 1) {
+        hipLaunchKernelGGL((attn_decode_worker<D, CL, T>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64), 0, stream, p);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (p.kernel_mask & 2) hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -168,6 +168,7 @@ struct AttnParams {
     int32_t B, H, G, R, Tq, KV_CTX;
     int32_t W, phase, stage, qwin;
     int32_t NW;  // number of decode workers (waves) the key tiles are dealt to
+    int32_t kernel_mask;  // bit 0: main kernel, bit 1: merge kernel
     float c;     // softmax scale * log2(e)
 };
 

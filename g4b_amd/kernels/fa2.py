@@ -77,6 +77,7 @@ def flash_attention(
     window_sizes=None,
     workspace=None,
     num_workers: int = 0,
+    kernel_mask: int = 0,
     stream=None,
 ):
     """``o[b, h, i] = softmax(scale * q[b, h, i] . K_b^T + mask) V_b`` for every in-phase slot ``b``.
@@ -102,7 +103,8 @@ def flash_attention(
     * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
       ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
       ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
-      used for split partials instead of the private one); ``num_workers``; ``stream``.
+      used for split partials instead of the private one); ``num_workers``; ``kernel_mask`` (profiling:
+      bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
 
     Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
     ignore (``g4b/models/gemma4e.py:593-607``).
@@ -170,6 +172,7 @@ def flash_attention(
     if query_window is not None and a.query_window < 1:
         raise ValueError("query_window must be a positive int or None")
     a.num_workers = int(num_workers)
+    a.kernel_mask = int(kernel_mask)
     a.scale = float(scale)
 
     ws = workspace

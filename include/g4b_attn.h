@@ -65,6 +65,9 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *                 Contents are unspecified after the call (like partial_o/l/m, fa2.py:643-645).
  *   num_workers   0 = library default; otherwise the number of waves the decode key tiles are
  *                 dealt to (must not exceed the value the workspace was sized for).
+ *   kernel_mask   profiling aid.  0 = run every kernel of the launch.  Otherwise bit 0 selects the
+ *                 main attention kernel and bit 1 the split-merge kernel of a decode-shaped launch,
+ *                 so that each can be timed on its own; results are only complete with both.
  *
  * Rows whose visible key set is empty (time_dim_sizes[b] == 0 on an in-phase slot) are written
  * as zeros; the reference leaves 0/0 there and its caller ignores them (g4b/scheduler.py:142-148).
@@ -95,6 +98,7 @@ typedef struct g4b_attn_args {
     int32_t stage;
     int32_t query_window;
     int32_t num_workers;
+    int32_t kernel_mask;
     float scale;
 } g4b_attn_args;
 

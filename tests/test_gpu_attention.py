@@ -53,8 +53,9 @@ def test_decode_matches_oracle_split_and_unsplit(fa, case, scale):
     fa.flash_attention(q, k, v, o2, i32(tds), u8(phase), W, ix.PHASE_DECODE, *partials(4, B, H, 1, D), scale=scale)
     torch.cuda.synchronize()
     assert_close(o2.float().cpu().numpy(), ref, what=f"{name} split")
-    # split and unsplit agree far inside the tolerance (test_fa2.py:432-433)
-    assert (o2.float() - o.float()).abs().max().item() < 1e-3
+    # split and unsplit agree to an fp16 ulp or two of the output (test_fa2.py:432-433 prints this difference)
+    diff = (o2.float() - o.float()).abs()
+    assert bool((diff <= 5e-4 + 2e-3 * o.float().abs()).all()), diff.max().item()
 
 
 @pytest.mark.parametrize("num_workers", [1, 3, 64, 777, 4096])

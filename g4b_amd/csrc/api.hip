@@ -65,7 +65,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         return fail(G4B_ERR_INVALID_ARGUMENT, "stage must be STAGE_FULL (1) or STAGE_CAUSAL (3), got %d", a->stage);
     if (a->phase < 0 || a->phase > 255) return fail(G4B_ERR_INVALID_ARGUMENT, "phase must fit uint8");
     if (a->query_window < 0) return fail(G4B_ERR_INVALID_ARGUMENT, "query_window must be >= 0");
-    if (!std::isfinite(a->scale)) return fail(G4B_ERR_INVALID_ARGUMENT, "scale must be finite");
+    if (!std::isfinite(a->scale) || !(a->scale > 0.f)) return fail(G4B_ERR_INVALID_ARGUMENT, "scale must be finite and positive");
     if (a->q_stride[3] != 1 || a->o_stride[3] != 1)
         return fail(G4B_ERR_INVALID_ARGUMENT, "q and o must have unit stride in the head dimension");
     for (int i = 0; i < 3; ++i)

@@ -5,16 +5,22 @@
 // group.  Each wave owns 32 rows.  The KV loop walks 64-key tiles from the first tile any row
 // of the workgroup can see to the causal diagonal; tiles entirely inside every row's range run
 // without masks, edge tiles (sliding-window lower edge, causal diagonal, window end) compare
-// per element.  Tiles are double-buffered in LDS: K row-major with a 16-byte row pad, V
-// transposed ([d][key]) with an XOR swizzle of the 16-byte column groups, both read back with
-// conflict-free ds_read_b128 in MFMA operand layout.
+// per element.
+//
+// Staging.  Tiles are double-buffered in LDS.  K goes global -> LDS directly
+// (global_load_lds_dwordx4, no registers): rows stay row-major and unpadded, the 16-byte pieces
+// of a row are XOR-swizzled with (row & 7) by choosing which global piece each lane fetches.
+// V passes through registers for an in-lane 8x8 16-bit transpose and is stored as V^T
+// ([d][key], 128-byte rows) with the 16-byte column groups XOR-swizzled.  Both are read back
+// with conflict-free ds_read_b128 directly in MFMA operand layout.
 //
 // Math per tile and wave: S^T[64 keys x 32 rows] = K Q^T and O^T[D x 32 rows] += V^T P on
 // v_mfma_f32_32x32x16 (fp16 or bf16 operands, fp32 accumulate).  Q stays in registers as the B
 // operand; P never leaves registers: the accumulator layout of S^T is the B-operand layout of
 // the second product once the key order inside each 16-key group of V^T is permuted to match.
-// Softmax is online in fp32 with exp2 and scale*log2(e) folded into one multiplier; the row
-// statistics live one row per lane pair (lane, lane^32).
+// LDS operand reads run a fixed number of steps ahead of the MFMAs that consume them.
+// Softmax is online in fp32 with exp2 and scale*log2(e) folded into one FMA; the row statistics
+// live one row per lane pair (lane, lane^32).
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -22,15 +28,20 @@ namespace g4b {
 
 constexpr int PF_BM = 128;  // query rows per workgroup
 constexpr int PF_BN = 64;   // keys per tile
+constexpr int PF_PD = 4;    // LDS operand reads in flight ahead of the MFMA that uses them
+constexpr float PF_TAU = 8.f;  // log2 of the growth of a row maximum that triggers a rescale
 
 template <int D>
 struct PfSmem {
-    static constexpr int KROW = D * 2 + 16;  // bytes per K row in LDS
+    static constexpr int KROW = D * 2;  // bytes per K row in LDS (unpadded, swizzled)
     static constexpr int KBYTES = PF_BN * KROW;
-    static constexpr int VROW = PF_BN * 2;  // bytes per V^T row (64 keys), swizzled, unpadded
+    static constexpr int VROW = PF_BN * 2;  // bytes per V^T row (64 keys), swizzled
     static constexpr int VBYTES = D * VROW;
     static constexpr int STAGE = KBYTES + VBYTES;
 };
+
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
 
 template <int D, class T>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
@@ -38,11 +49,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     extern __shared__ __align__(16) char smem[];
     constexpr int KSTEPS = D / 16;  // contraction steps of the first product
     constexpr int DT = D / 32;      // 32-row tiles of O^T
-    constexpr int PIECES = D / 8;   // 16-byte pieces per cache row
-    constexpr int KLD = PF_BN * PIECES / 256;  // 16-byte K loads per thread and tile
-    constexpr int VSEG = D / 8;                // 8-wide d segments per row
-    constexpr int VITEMS = (PF_BN / 8) * VSEG;     // (8-key group, d segment) items per tile
-    constexpr int VLD = (VITEMS + 255) / 256;      // items per thread
+    constexpr int KCHUNKS = SM::KBYTES / 1024 / 4;  // 1 KiB direct-to-LDS loads per wave and tile
+    constexpr int ROWS_PER_CHUNK = 1024 / SM::KROW;
+    constexpr int PIECES = D / 8;
+    constexpr int VSEG = D / 8;                 // 8-wide d segments per row
+    constexpr int VITEMS = (PF_BN / 8) * VSEG;  // (8-key group, d segment) items per tile
+    static_assert(VITEMS <= 256, "one V item per thread");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -58,10 +70,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     const int tok0 = qtile * TOKB;
     const int tok_last = min(tok0 + TOKB, Tq) - 1;
     // key range of the workgroup and the range that every row shares
-    int lo_wg, hi_wg, lo_max, hi_min, dummy;
+    int lo_wg, hi_wg, lo_max, hi_min;
     row_range(p, si, tok0, lo_wg, hi_min);
     row_range(p, si, tok_last, lo_max, hi_wg);
-    (void)dummy;
 
     // this lane's row
     const int rrow = wave * 32 + n32;
@@ -79,7 +90,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     for (int i = 0; i < DT; ++i)
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;  // running max in log2 units (scaled), running sum (this lane's keys)
 
     if (hi_wg > lo_wg) {
         // Q as B operand: lane (row n32, half h2), step c: d = 16c + 8*h2 .. +8
@@ -99,97 +110,150 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             return (uint32_t)r * (uint32_t)(D * 2);
         };
 
-        // staging roles
-        const int k_piece = tid % PIECES, k_row0 = tid / PIECES;  // rows k_row0 + (256/PIECES)*i
-        constexpr int KROWSTEP = 256 / PIECES;
+        // ---- staging roles ------------------------------------------------------------------------
+        // K: wave `wave` issues KCHUNKS direct loads; chunk c covers LDS bytes [c*1024, +1024) of the K tile.
+        const int k_row_in_chunk = lane / PIECES;  // 0 .. ROWS_PER_CHUNK-1
+        const int k_piece_lds = lane % PIECES;
+        // V: thread item = (8-key group q8, d segment)
+        const int v_q8 = tid / VSEG, v_dseg = tid % VSEG;
+        const bool v_item = (VITEMS == 256) || tid < VITEMS;
+        u4 vst[8];
 
-        u4 kst[KLD];
-        u4 vst[VLD][8];
-        auto load_tile = [&](int kt) {
+        auto issue_k = [&](int kt, int stage) {
             const int jb = kt * PF_BN;
+            char* ks = smem + stage * SM::STAGE;
 #pragma unroll
-            for (int i = 0; i < KLD; ++i) kst[i] = ld16(kbase, key_off(jb + k_row0 + KROWSTEP * i) + (uint32_t)k_piece * 16u);
-#pragma unroll
-            for (int it = 0; it < VLD; ++it) {
-                const int item = tid + 256 * it;
-                const int q8 = item / VSEG, dseg = item % VSEG;
-                // 8-key group q8 of the tile: 16-key group q8/2, half hsel = q8 & 1; slot j -> key 8*(j/4) + 4*hsel + j%4
-                const int kb16 = jb + (q8 >> 1) * 16 + (q8 & 1) * 4;
-                if (item < VITEMS) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        vst[it][j] = ld16(vbase, key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)dseg * 16u);
-                }
+            for (int i = 0; i < KCHUNKS; ++i) {
+                const int chunk = wave * KCHUNKS + i;
+                const int row = chunk * ROWS_PER_CHUNK + k_row_in_chunk;
+                const int piece = k_piece_lds ^ (row & 7);
+                const char* src = kbase + key_off(jb + row) + (uint32_t)piece * 16u;
+                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ks + chunk * 1024), 16, 0, 0);
             }
         };
-        auto store_tile = [&](int stage) {
-            char* ks = smem + stage * SM::STAGE;
-            char* vs = ks + SM::KBYTES;
+        auto issue_v = [&](int kt) {
+            const int jb = kt * PF_BN;
+            // 8-key group q8: 16-key group q8/2, half q8 & 1; slot j -> key 8*(j/4) + 4*half + j%4
+            const int kb16 = jb + (v_q8 >> 1) * 16 + (v_q8 & 1) * 4;
+            if (v_item) {
 #pragma unroll
-            for (int i = 0; i < KLD; ++i)
-                *reinterpret_cast<u4*>(ks + (k_row0 + KROWSTEP * i) * SM::KROW + k_piece * 16) = kst[i];
-#pragma unroll
-            for (int it = 0; it < VLD; ++it) {
-                const int item = tid + 256 * it;
-                const int q8 = item / VSEG, dseg = item % VSEG;
-                if (item >= VITEMS) continue;
+                for (int j = 0; j < 8; ++j)
+                    vst[j] = ld16(vbase, key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)v_dseg * 16u);
+            }
+        };
+        auto store_v = [&](int stage) {
+            char* vs = smem + stage * SM::STAGE + SM::KBYTES;
+            if (v_item) {
                 u4 vt[8];
-                transpose8x8_b16(vst[it], vt);
+                transpose8x8_b16(vst, vt);
 #pragma unroll
                 for (int jj = 0; jj < 8; ++jj) {
-                    const int d = dseg * 8 + jj;
-                    const int slot = q8 ^ ((d ^ (d >> 3)) & 7);
+                    const int d = v_dseg * 8 + jj;
+                    const int slot = v_q8 ^ ((jj ^ v_dseg) & 7);
                     *reinterpret_cast<u4*>(vs + d * SM::VROW + slot * 16) = vt[jj];
                 }
             }
         };
 
+        // ---- operand read offsets (bytes inside a stage) -----------------------------------------
+        // K^T step (mt, c): row mt*32 + n32, piece 2c + h2, swizzled with (row & 7) = (n32 & 7)
+        uint32_t koff[4];
+#pragma unroll
+        for (int c4 = 0; c4 < 4; ++c4) koff[c4] = (uint32_t)n32 * SM::KROW + (uint32_t)(((2 * c4 + h2) ^ (n32 & 7)) * 16);
+        // V^T step (dt, mt, u): row d = 32*dt + n32, column group (4*mt + 2*u + h2) ^ swz(d)
+        uint32_t voff[2][4];
+#pragma unroll
+        for (int par = 0; par < 2; ++par) {
+            const int d = par * 32 + n32;
+            const int sw = (d ^ (d >> 3)) & 7;
+#pragma unroll
+            for (int cu = 0; cu < 4; ++cu) voff[par][cu] = SM::KBYTES + (uint32_t)n32 * SM::VROW + (uint32_t)(((2 * cu + h2) ^ sw) * 16);
+        }
+
         const int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
-        load_tile(kt0);
-        store_tile(0);
+        issue_k(kt0, 0);
+        issue_v(kt0);
+        store_v(0);
         __syncthreads();
 
         for (int kt = kt0; kt <= kt1; ++kt) {
             const int stage = (kt - kt0) & 1;
-            const char* ks = smem + stage * SM::STAGE;
-            const char* vs = ks + SM::KBYTES;
-            if (kt < kt1) load_tile(kt + 1);
+            const char* sb = smem + stage * SM::STAGE;
+            // the tile after the last one is fetched too (addresses are clamped to the window); nobody reads it
+            issue_k(kt + 1, stage ^ 1);
+            issue_v(kt + 1);
 
-            // ---- S^T = K Q^T : 2 key tiles of 32 -------------------------------------------
+            // ---- S^T = K Q^T : two 32-key tiles, interleaved so consecutive MFMAs are independent ----
             f16v s[2];
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
+            for (int j = 0; j < 16; ++j) {
+                s[0][j] = 0.f;
+                s[1][j] = 0.f;
+            }
+            {
+                constexpr int NSTEP = 2 * KSTEPS;
+                auto rd = [&](int idx) -> u4 {
+                    const int c = idx >> 1, mt = idx & 1;
+                    return *reinterpret_cast<const u4*>(sb + koff[c & 3] + (uint32_t)(mt * 32 * SM::KROW + (c >> 2) * 128));
+                };
+                u4 abuf[PF_PD];
 #pragma unroll
-                for (int j = 0; j < 16; ++j) s[mt][j] = 0.f;
-                const char* krow = ks + (mt * 32 + n32) * SM::KROW + h2 * 16;
+                for (int i = 0; i < PF_PD; ++i) abuf[i] = rd(i);
 #pragma unroll
-                for (int c = 0; c < KSTEPS; ++c) {
-                    const u4 a = *reinterpret_cast<const u4*>(krow + c * 32);
-                    s[mt] = T::mfma32(a, qf[c], s[mt]);
+                for (int idx = 0; idx < NSTEP; ++idx) {
+                    const u4 a = abuf[idx % PF_PD];
+                    if (idx + PF_PD < NSTEP) abuf[idx % PF_PD] = rd(idx + PF_PD);
+                    s[idx & 1] = T::mfma32(a, qf[idx >> 1], s[idx & 1]);
                 }
+                __builtin_amdgcn_sched_group_barrier(0x100, PF_PD, 0);
+#pragma unroll
+                for (int idx = 0; idx < NSTEP - PF_PD; ++idx) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, PF_PD, 0);
             }
 
             // ---- online softmax ---------------------------------------------------------------
             const int jb = kt * PF_BN;
-            const bool edge = (jb < lo_max) || (jb + PF_BN > hi_min);
-            float mx = -INFINITY;
+            if ((jb < lo_max) || (jb + PF_BN > hi_min)) {
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+                for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    float x = s[mt][i] * p.c;
-                    if (edge) {
+                    for (int i = 0; i < 16; ++i) {
                         const int j = jb + mt * 32 + 8 * (i >> 2) + 4 * h2 + (i & 3);
-                        if (j < lo_r || j >= hi_r) x = -INFINITY;
+                        if (j < lo_r || j >= hi_r) s[mt][i] = -INFINITY;
                     }
-                    s[mt][i] = x;
-                    mx = fmaxf(mx, x);
+            }
+            float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
+            mx = fmaxf(mx, __shfl_xor(mx, 32)) * p.c;  // scale > 0: max commutes with the scaling
+            // Lazy rescaling: the reference point m_run of the exponentials only moves when the row maximum
+            // outgrows it by more than 2^PF_TAU, so P stays below 2^PF_TAU and the accumulators are rarely touched.
+            const bool grow = mx > m_run + PF_TAU;
+            if (__any(grow)) {
+                const float m_new = grow ? mx : m_run;
+                const float alpha = grow ? fast_exp2(m_run - mx) : 1.f;  // 0 on a row's first keys
+                const bool touch = grow && (m_run != -INFINITY);
+                m_run = m_new;
+                l_run *= alpha;
+                if (__any(touch)) {
+                    // The accumulators live in AGPRs.  Spelling the read-scale-write out keeps the copies inside
+                    // this rarely taken branch instead of on the main path.
+#pragma unroll
+                    for (int i = 0; i < DT; ++i)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) {
+                            float t, r;
+                            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[i][j]));
+                            t *= alpha;
+                            asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(r) : "v"(t));
+                            acc[i][j] = r;
+                        }
                 }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run, mx);
-            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = fast_exp2(m_run - m_safe);
-            m_run = m_new;
+            }
+            const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
             float psum = 0.f;
             u4 pf[2][2];  // [key tile][16-key group] -> 8 keys of this lane half
 #pragma unroll
@@ -199,34 +263,40 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                     float e[8];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        e[j] = fast_exp2(s[mt][8 * u + j] - m_safe);
+                        e[j] = fast_exp2(__builtin_fmaf(s[mt][8 * u + j], p.c, -m_safe));
                         psum += e[j];
                     }
                     pf[mt][u] = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
                 }
-            l_run = l_run * alpha + psum;
-            if (__any(alpha != 1.f)) {
+            l_run += psum;
+
+            // ---- O^T += V^T P : (key group) outer, d tile inner -> consecutive MFMAs are independent ----
+            {
+                constexpr int NSTEP = 4 * DT;
+                auto rd = [&](int idx) -> u4 {
+                    const int cu = idx / DT, dt = idx % DT;
+                    return *reinterpret_cast<const u4*>(sb + voff[dt & 1][cu] + (uint32_t)(dt * 32 * SM::VROW));
+                };
+                u4 abuf[PF_PD];
 #pragma unroll
-                for (int i = 0; i < DT; ++i) acc[i] *= alpha;
+                for (int i = 0; i < PF_PD; ++i) abuf[i] = rd(i);
+#pragma unroll
+                for (int idx = 0; idx < NSTEP; ++idx) {
+                    const u4 a = abuf[idx % PF_PD];
+                    if (idx + PF_PD < NSTEP) abuf[idx % PF_PD] = rd(idx + PF_PD);
+                    const int cu = idx / DT, dt = idx % DT;
+                    acc[dt] = T::mfma32(a, pf[cu >> 1][cu & 1], acc[dt]);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, PF_PD, 1);
+#pragma unroll
+                for (int idx = 0; idx < NSTEP - PF_PD; ++idx) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, PF_PD, 1);
             }
 
-            // ---- O^T += V^T P -------------------------------------------------------------------
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const int d = dt * 32 + n32;
-                const int sw = (d ^ (d >> 3)) & 7;
-                const char* vrow = vs + d * SM::VROW;
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        const int slot = (mt * 4 + u * 2 + h2) ^ sw;
-                        const u4 a = *reinterpret_cast<const u4*>(vrow + slot * 16);
-                        acc[dt] = T::mfma32(a, pf[mt][u], acc[dt]);
-                    }
-            }
-
-            if (kt < kt1) store_tile(stage ^ 1);
+            store_v(stage ^ 1);
             __syncthreads();
         }
     }

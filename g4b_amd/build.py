@@ -26,7 +26,7 @@ SOURCES = ["api.hip", "attn_decode.hip", "attn_prefill.hip", "cache_ops.hip"]
 
 # packed-fp32 VALU forms are kept off: the compiler must not form v_pk_{add,mul,fma}_f32
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-variable", "-Wno-unknown-pragmas"]
+COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-variable", "-Wno-unknown-pragmas"]
 
 
 def hipcc() -> str:

@@ -9,7 +9,7 @@
 //
 // Staging.  Tiles are double-buffered in LDS.  K goes global -> LDS directly
 // (global_load_lds_dwordx4, no registers): rows stay row-major and unpadded, the 16-byte pieces
-// of a row are XOR-swizzled with (row & 7) by choosing which global piece each lane fetches.
+// of a row are XOR-swizzled with (row & 15) by choosing which global piece each lane fetches.
 // V passes through registers for an in-lane 8x8 16-bit transpose and is stored as V^T
 // ([d][key], 128-byte rows) with the 16-byte column groups XOR-swizzled.  Both are read back
 // with conflict-free ds_read_b128 directly in MFMA operand layout.
@@ -121,12 +121,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 
         auto issue_k = [&](int kt, int stage) {
             const int jb = kt * PF_BN;
-            char* ks = smem + stage * SM::STAGE;
+            char* ks = smem + stage * SM::KBYTES;
 #pragma unroll
             for (int i = 0; i < KCHUNKS; ++i) {
                 const int chunk = wave * KCHUNKS + i;
                 const int row = chunk * ROWS_PER_CHUNK + k_row_in_chunk;
-                const int piece = k_piece_lds ^ (row & 7);
+                const int piece = k_piece_lds ^ (row & 15);
                 const char* src = kbase + key_off(jb + row) + (uint32_t)piece * 16u;
                 __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ks + chunk * 1024), 16, 0, 0);
             }
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             }
         };
         auto store_v = [&](int stage) {
-            char* vs = smem + stage * SM::STAGE + SM::KBYTES;
+            char* vs = smem + 2 * SM::KBYTES + stage * SM::VBYTES;
             if (v_item) {
                 u4 vt[8];
                 transpose8x8_b16(vst, vt);
@@ -155,11 +155,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             }
         };
 
-        // ---- operand read offsets (bytes inside a stage) -----------------------------------------
-        // K^T step (mt, c): row mt*32 + n32, piece 2c + h2, swizzled with (row & 7) = (n32 & 7)
-        uint32_t koff[4];
+        // ---- operand read offsets ------------------------------------------------------------------
+        // LDS map: K stages at [0, 2*KBYTES), V^T stages at [2*KBYTES, 2*KBYTES + 2*VBYTES).
+        // K^T step (mt, c): row mt*32 + n32, piece 2c + h2, swizzled with (row & 15) = (n32 & 15)
+        uint32_t koff[8];
 #pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) koff[c4] = (uint32_t)n32 * SM::KROW + (uint32_t)(((2 * c4 + h2) ^ (n32 & 7)) * 16);
+        for (int c8 = 0; c8 < 8; ++c8) koff[c8] = (uint32_t)n32 * SM::KROW + (uint32_t)(((2 * c8 + h2) ^ (n32 & 15)) * 16);
         // V^T step (dt, mt, u): row d = 32*dt + n32, column group (4*mt + 2*u + h2) ^ swz(d)
         uint32_t voff[2][4];
 #pragma unroll
@@ -167,54 +168,83 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             const int d = par * 32 + n32;
             const int sw = (d ^ (d >> 3)) & 7;
 #pragma unroll
-            for (int cu = 0; cu < 4; ++cu) voff[par][cu] = SM::KBYTES + (uint32_t)n32 * SM::VROW + (uint32_t)(((2 * cu + h2) ^ sw) * 16);
+            for (int cu = 0; cu < 4; ++cu) voff[par][cu] = 2 * SM::KBYTES + (uint32_t)n32 * SM::VROW + (uint32_t)(((2 * cu + h2) ^ sw) * 16);
         }
+        constexpr int QK_STEPS = 2 * KSTEPS;  // MFMAs of S^T = K Q^T per tile; step idx -> (c = idx/2, key tile mt = idx%2)
+        constexpr int PV_STEPS = 4 * DT;      // MFMAs of O^T += V^T P per tile; step idx -> (key group idx/DT, d tile idx%DT)
+        const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the dynamic segment
+        // Operand reads are issued as volatile asm, PF_PD steps ahead of the MFMA that consumes them, and
+        // retired with explicit lgkmcnt waits: LDS returns data in order, so "at most n outstanding" is exact
+        // for the oldest read whatever else the compiler has in flight.
+        uint32_t kaddr[8], vaddr[2][4];
+        // `left` = reads of the same sequence issued after the one being retired (a constant after unrolling)
+        auto wait_left = [&](u4& a, int left) {
+            static_assert(PF_PD == 4, "wait ladder below is written for 4 reads in flight");
+            if (left >= 3) lds_wait<3>(a);
+            else if (left == 2) lds_wait<2>(a);
+            else if (left == 1) lds_wait<1>(a);
+            else lds_wait<0>(a);
+        };
+        auto k_issue = [&](int idx) -> u4 {  // needs kaddr[] of the stage
+            const int c = idx >> 1, mt = idx & 1;
+            return lds_read16(kaddr[c & 7], mt * 32 * SM::KROW + (c >> 3) * 256);
+        };
+        auto v_issue = [&](int idx) -> u4 {
+            const int cu = idx / DT, dt = idx % DT;
+            return lds_read16(vaddr[dt & 1][cu], dt * 32 * SM::VROW);
+        };
 
         const int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
+
+        // ---- prologue: K(kt0), K(kt0+1), V(kt0) staged; S(kt0) computed --------------------------------
         issue_k(kt0, 0);
+        issue_k(kt0 + 1, 1);
         issue_v(kt0);
         store_v(0);
         __syncthreads();
+        f16v s_cur[2];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            s_cur[0][j] = 0.f;
+            s_cur[1][j] = 0.f;
+        }
+        {
+#pragma unroll
+            for (int c8 = 0; c8 < 8; ++c8) kaddr[c8] = lds0 + koff[c8];
+            u4 abuf[PF_PD];
+#pragma unroll
+            for (int i = 0; i < PF_PD; ++i) abuf[i] = k_issue(i);
+#pragma unroll
+            for (int idx = 0; idx < QK_STEPS; ++idx) {
+                u4 a = abuf[idx % PF_PD];
+                wait_left(a, QK_STEPS - 1 - idx);
+                if (idx + PF_PD < QK_STEPS) abuf[idx % PF_PD] = k_issue(idx + PF_PD);
+                s_cur[idx & 1] = T::mfma32(a, qf[idx >> 1], s_cur[idx & 1]);
+            }
+        }
+        __syncthreads();  // every wave is done with K stage 0 before the loop refills it
 
+        // One tile: softmax of S(kt) and O += V(kt) P, overlapped with S(kt+1) = K(kt+1) Q^T.
+        // par = (kt - kt0) & 1: V(kt) sits in V stage par, K(kt+1) in K stage par^1; K(kt+2) is fetched into K
+        // stage par and V(kt+1) into V stage par^1 while this tile computes.
         for (int kt = kt0; kt <= kt1; ++kt) {
-            const int stage = (kt - kt0) & 1;
-            const char* sb = smem + stage * SM::STAGE;
-            // the tile after the last one is fetched too (addresses are clamped to the window); nobody reads it
-            issue_k(kt + 1, stage ^ 1);
+            constexpr int N1 = 8;  // QK steps issued next to the row-max part of the softmax
+            const int par = (kt - kt0) & 1;
+            // the tiles after the last one are fetched (addresses are clamped to the window) and multiplied too;
+            // nobody reads the results
+            issue_k(kt + 2, par);
             issue_v(kt + 1);
-
-            // ---- S^T = K Q^T : two 32-key tiles, interleaved so consecutive MFMAs are independent ----
-            f16v s[2];
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                s[0][j] = 0.f;
-                s[1][j] = 0.f;
-            }
             {
-                constexpr int NSTEP = 2 * KSTEPS;
-                auto rd = [&](int idx) -> u4 {
-                    const int c = idx >> 1, mt = idx & 1;
-                    return *reinterpret_cast<const u4*>(sb + koff[c & 3] + (uint32_t)(mt * 32 * SM::KROW + (c >> 2) * 128));
-                };
-                u4 abuf[PF_PD];
+                const uint32_t kb = lds0 + (par ^ 1) * SM::KBYTES, vb = lds0 + par * SM::VBYTES;
 #pragma unroll
-                for (int i = 0; i < PF_PD; ++i) abuf[i] = rd(i);
+                for (int c8 = 0; c8 < 8; ++c8) kaddr[c8] = kb + koff[c8];
 #pragma unroll
-                for (int idx = 0; idx < NSTEP; ++idx) {
-                    const u4 a = abuf[idx % PF_PD];
-                    if (idx + PF_PD < NSTEP) abuf[idx % PF_PD] = rd(idx + PF_PD);
-                    s[idx & 1] = T::mfma32(a, qf[idx >> 1], s[idx & 1]);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x100, PF_PD, 0);
+                for (int q = 0; q < 2; ++q)
 #pragma unroll
-                for (int idx = 0; idx < NSTEP - PF_PD; ++idx) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, PF_PD, 0);
+                    for (int cu = 0; cu < 4; ++cu) vaddr[q][cu] = vb + voff[q][cu];  // voff includes the 2*KBYTES base
             }
 
-            // ---- online softmax ---------------------------------------------------------------
+            // ---- edge tiles only: mask S(kt) before anything else so the rest of the tile is one straight block
             const int jb = kt * PF_BN;
             if ((jb < lo_max) || (jb + PF_BN > hi_min)) {
 #pragma unroll
@@ -222,13 +252,34 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int j = jb + mt * 32 + 8 * (i >> 2) + 4 * h2 + (i & 3);
-                        if (j < lo_r || j >= hi_r) s[mt][i] = -INFINITY;
+                        if (j < lo_r || j >= hi_r) s_cur[mt][i] = -INFINITY;
                     }
             }
-            float mx = fmaxf(s[0][0], s[1][0]);
+
+            f16v s_nxt[2];
+            u4 abuf[PF_PD];
 #pragma unroll
-            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
-            mx = fmaxf(mx, __shfl_xor(mx, 32)) * p.c;  // scale > 0: max commutes with the scaling
+            for (int j = 0; j < 16; ++j) {
+                s_nxt[0][j] = 0.f;
+                s_nxt[1][j] = 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < PF_PD; ++i) abuf[i] = k_issue(i);
+            auto qk_step = [&](int idx) {
+                u4 a = abuf[idx % PF_PD];
+                wait_left(a, QK_STEPS - 1 - idx);
+                if (idx + PF_PD < QK_STEPS) abuf[idx % PF_PD] = k_issue(idx + PF_PD);
+                s_nxt[idx & 1] = T::mfma32(a, qf[idx >> 1], s_nxt[idx & 1]);
+            };
+#pragma unroll
+            for (int idx = 0; idx < N1; ++idx) qk_step(idx);
+
+            // ---- softmax, part 1: row maximum --------------------------------------------------------------
+            float mx = fmaxf(s_cur[0][0], s_cur[1][0]);
+#pragma unroll
+            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s_cur[0][i], s_cur[1][i]));
+            mx = half_swap_max(mx) * p.c;  // scale > 0: max commutes with the scaling
+
             // Lazy rescaling: the reference point m_run of the exponentials only moves when the row maximum
             // outgrows it by more than 2^PF_TAU, so P stays below 2^PF_TAU and the accumulators are rarely touched.
             const bool grow = mx > m_run + PF_TAU;
@@ -253,6 +304,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                         }
                 }
             }
+
+            // ---- softmax, part 2: exponentials, row sums, P in MFMA operand layout ---------------------------
             const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
             float psum = 0.f;
             u4 pf[2][2];  // [key tile][16-key group] -> 8 keys of this lane half
@@ -263,41 +316,34 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                     float e[8];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        e[j] = fast_exp2(__builtin_fmaf(s[mt][8 * u + j], p.c, -m_safe));
+                        e[j] = fast_exp2(__builtin_fmaf(s_cur[mt][8 * u + j], p.c, -m_safe));
                         psum += e[j];
                     }
                     pf[mt][u] = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
+                    // six of the remaining K Q^T steps next to each quarter of the exponentials
+#pragma unroll
+                    for (int q = 0; q < (QK_STEPS - N1) / 4; ++q) qk_step(N1 + (mt * 2 + u) * ((QK_STEPS - N1) / 4) + q);
                 }
             l_run += psum;
 
-            // ---- O^T += V^T P : (key group) outer, d tile inner -> consecutive MFMAs are independent ----
+            // ---- O^T += V^T P : (key group) outer, d tile inner -> consecutive MFMAs are independent ----------
             {
-                constexpr int NSTEP = 4 * DT;
-                auto rd = [&](int idx) -> u4 {
-                    const int cu = idx / DT, dt = idx % DT;
-                    return *reinterpret_cast<const u4*>(sb + voff[dt & 1][cu] + (uint32_t)(dt * 32 * SM::VROW));
-                };
-                u4 abuf[PF_PD];
+                u4 vbuf[PF_PD];
 #pragma unroll
-                for (int i = 0; i < PF_PD; ++i) abuf[i] = rd(i);
+                for (int i = 0; i < PF_PD; ++i) vbuf[i] = v_issue(i);
 #pragma unroll
-                for (int idx = 0; idx < NSTEP; ++idx) {
-                    const u4 a = abuf[idx % PF_PD];
-                    if (idx + PF_PD < NSTEP) abuf[idx % PF_PD] = rd(idx + PF_PD);
+                for (int idx = 0; idx < PV_STEPS; ++idx) {
+                    u4 a = vbuf[idx % PF_PD];
+                    wait_left(a, PV_STEPS - 1 - idx);
+                    if (idx + PF_PD < PV_STEPS) vbuf[idx % PF_PD] = v_issue(idx + PF_PD);
                     const int cu = idx / DT, dt = idx % DT;
                     acc[dt] = T::mfma32(a, pf[cu >> 1][cu & 1], acc[dt]);
                 }
-                __builtin_amdgcn_sched_group_barrier(0x100, PF_PD, 1);
-#pragma unroll
-                for (int idx = 0; idx < NSTEP - PF_PD; ++idx) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, PF_PD, 1);
             }
-
-            store_v(stage ^ 1);
+            store_v(par ^ 1);
             __syncthreads();
+            s_cur[0] = s_nxt[0];
+            s_cur[1] = s_nxt[1];
         }
     }
 

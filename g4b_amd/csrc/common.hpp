@@ -137,6 +137,35 @@ G4B_DEV int wave_incl_scan_i(int v, int lane) {
 
 G4B_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// max / sum over the lane pair (l, l ^ 32) without going through LDS: v_permlane32_swap exchanges the upper half
+// of its first operand with the lower half of its second, leaving (low half, low half) and (high half, high half).
+// The two results are copied into scalars before the bit casts: __builtin_bit_cast applied directly to an element of
+// an ext_vector reads element 0 whatever the index.
+G4B_DEV float half_swap_max(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    const u2 r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+G4B_DEV float half_swap_sum(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    const u2 r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+// 16-byte LDS read issued where it is written (volatile asm), to be retired by lds_wait<n> on the same value.
+G4B_DEV u4 lds_read16(uint32_t lds_addr, int imm) {
+    u4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(imm));
+    return v;
+}
+// Wait until at most N LDS operations are outstanding; v is tied so its consumers stay behind the wait.
+template <int N>
+G4B_DEV void lds_wait(u4& v) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
+}
+
 // In-lane 8x8 transpose of 16-bit elements.  in[s] holds elements (s, 0..7); out[j] holds (0..7, j).
 G4B_DEV void transpose8x8_b16(const u4 (&in)[8], u4 (&out)[8]) {
 #pragma unroll

@@ -119,26 +119,62 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
         const bool v_item = (VITEMS == 256) || tid < VITEMS;
         u4 vst[8];
 
+        // A tile is "plain" when its 64 keys lie inside the window and do not straddle the ring seam: then its rows
+        // are consecutive in memory and every lane's source offset is a loop constant added to one scalar base.
+        // Only the first / last tiles of a slot and the one on the seam take the general path with per-row clamping.
+        uint32_t k_const[KCHUNKS], v_const[8];
+#pragma unroll
+        for (int i = 0; i < KCHUNKS; ++i) {
+            const int row = (wave * KCHUNKS + i) * ROWS_PER_CHUNK + k_row_in_chunk;
+            k_const[i] = (uint32_t)row * SM::KROW + (uint32_t)(k_piece_lds ^ (row & 15)) * 16u;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            v_const[j] = (uint32_t)((v_q8 >> 1) * 16 + (v_q8 & 1) * 4 + 8 * (j >> 2) + (j & 3)) * SM::KROW + (uint32_t)v_dseg * 16u;
+        auto plain_row0 = [&](int kt) -> int {  // ring row of the tile's first key, or -1
+            const int jb = kt * PF_BN;
+            if (jb + PF_BN > si.window) return -1;
+            int r0 = si.ring_start + jb;
+            r0 = (r0 >= KV_CTX) ? r0 - KV_CTX : r0;
+            return (r0 + PF_BN <= KV_CTX) ? r0 : -1;
+        };
         auto issue_k = [&](int kt, int stage) {
             const int jb = kt * PF_BN;
             char* ks = smem + stage * SM::KBYTES;
+            const int r0 = plain_row0(kt);
+            if (r0 >= 0) {
+                const char* tb = kbase + (int64_t)r0 * SM::KROW;
 #pragma unroll
-            for (int i = 0; i < KCHUNKS; ++i) {
-                const int chunk = wave * KCHUNKS + i;
-                const int row = chunk * ROWS_PER_CHUNK + k_row_in_chunk;
-                const int piece = k_piece_lds ^ (row & 15);
-                const char* src = kbase + key_off(jb + row) + (uint32_t)piece * 16u;
-                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ks + chunk * 1024), 16, 0, 0);
+                for (int i = 0; i < KCHUNKS; ++i)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(tb + k_const[i]), (lptr_t)(ks + (wave * KCHUNKS + i) * 1024), 16, 0, 0);
+            } else {
+#pragma unroll
+                for (int i = 0; i < KCHUNKS; ++i) {
+                    const int chunk = wave * KCHUNKS + i;
+                    const int row = chunk * ROWS_PER_CHUNK + k_row_in_chunk;
+                    const int piece = k_piece_lds ^ (row & 15);
+                    const char* src = kbase + key_off(jb + row) + (uint32_t)piece * 16u;
+                    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ks + chunk * 1024), 16, 0, 0);
+                }
             }
         };
         auto issue_v = [&](int kt) {
             const int jb = kt * PF_BN;
-            // 8-key group q8: 16-key group q8/2, half q8 & 1; slot j -> key 8*(j/4) + 4*half + j%4
-            const int kb16 = jb + (v_q8 >> 1) * 16 + (v_q8 & 1) * 4;
-            if (v_item) {
+            const int r0 = plain_row0(kt);
+            if (r0 >= 0) {
+                const char* tb = vbase + (int64_t)r0 * SM::KROW;
+                if (v_item) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    vst[j] = ld16(vbase, key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)v_dseg * 16u);
+                    for (int j = 0; j < 8; ++j) vst[j] = ld16(tb, v_const[j]);
+                }
+            } else {
+                // 8-key group q8: 16-key group q8/2, half q8 & 1; slot j -> key 8*(j/4) + 4*half + j%4
+                const int kb16 = jb + (v_q8 >> 1) * 16 + (v_q8 & 1) * 4;
+                if (v_item) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        vst[j] = ld16(vbase, key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)v_dseg * 16u);
+                }
             }
         };
         auto store_v = [&](int stage) {
@@ -232,8 +268,36 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             const int par = (kt - kt0) & 1;
             // the tiles after the last one are fetched (addresses are clamped to the window) and multiplied too;
             // nobody reads the results
-            issue_k(kt + 2, par);
-            issue_v(kt + 1);
+            // Sources of K(kt+2) and V(kt+1): scalar base + per-lane offset (loop constants on plain tiles).  The
+            // loads themselves are issued a few at a time between the MFMA steps below so that the address unit is
+            // never handed more than one instruction per wave at once.
+            const char* ksrc = kbase;
+            const char* vsrc = vbase;
+            uint32_t kofs[KCHUNKS], vofs[8];
+            {
+                const int rk = plain_row0(kt + 2), rv = plain_row0(kt + 1);
+                if (rk >= 0) {
+                    ksrc = kbase + (int64_t)rk * SM::KROW;
+#pragma unroll
+                    for (int i = 0; i < KCHUNKS; ++i) kofs[i] = k_const[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KCHUNKS; ++i) {
+                        const int row = (wave * KCHUNKS + i) * ROWS_PER_CHUNK + k_row_in_chunk;
+                        kofs[i] = key_off((kt + 2) * PF_BN + row) + (uint32_t)(k_piece_lds ^ (row & 15)) * 16u;
+                    }
+                }
+                if (rv >= 0) {
+                    vsrc = vbase + (int64_t)rv * SM::KROW;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) vofs[j] = v_const[j];
+                } else {
+                    const int kb16 = (kt + 1) * PF_BN + (v_q8 >> 1) * 16 + (v_q8 & 1) * 4;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) vofs[j] = key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)v_dseg * 16u;
+                }
+            }
+            const uint32_t kdst = lds0 + par * SM::KBYTES + (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (KCHUNKS * 1024);
             {
                 const uint32_t kb = lds0 + (par ^ 1) * SM::KBYTES, vb = lds0 + par * SM::VBYTES;
 #pragma unroll
@@ -270,6 +334,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                 wait_left(a, QK_STEPS - 1 - idx);
                 if (idx + PF_PD < QK_STEPS) abuf[idx % PF_PD] = k_issue(idx + PF_PD);
                 s_nxt[idx & 1] = T::mfma32(a, qf[idx >> 1], s_nxt[idx & 1]);
+                // one of the eight V(kt+1) row loads every few steps of the second part
+                constexpr int VSTRIDE = (QK_STEPS - N1) / 8;
+                if (idx >= N1 && (idx - N1) % VSTRIDE == 0 && (idx - N1) / VSTRIDE < 8) {
+                    if (v_item) vst[(idx - N1) / VSTRIDE] = gload16_async(vsrc, vofs[(idx - N1) / VSTRIDE]);
+                }
             };
 #pragma unroll
             for (int idx = 0; idx < N1; ++idx) qk_step(idx);
@@ -338,9 +407,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                     if (idx + PF_PD < PV_STEPS) vbuf[idx % PF_PD] = v_issue(idx + PF_PD);
                     const int cu = idx / DT, dt = idx % DT;
                     acc[dt] = T::mfma32(a, pf[cu >> 1][cu & 1], acc[dt]);
+                    // one of the K(kt+2) direct-to-LDS loads every other step of the first half
+                    if (idx % 2 == 0 && idx / 2 < KCHUNKS) dma16_to_lds(ksrc, kofs[idx / 2], kdst + (idx / 2) * 1024);
                 }
             }
+            vm_wait8<KCHUNKS>(vst);  // the V loads were issued before the K loads
             store_v(par ^ 1);
+            vm_wait_all();
             __syncthreads();
             s_cur[0] = s_nxt[0];
             s_cur[1] = s_nxt[1];

@@ -160,6 +160,26 @@ G4B_DEV u4 lds_read16(uint32_t lds_addr, int imm) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(imm));
     return v;
 }
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16 * l (M0 carries the base).
+// Source address = scalar base + per-lane 32-bit offset.  Completion is tracked by vmcnt.
+G4B_DEV void dma16_to_lds(const void* sbase, uint32_t voff, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
+}
+// 16-byte global load issued where it is written; retire with vm_wait8 before the values are used.
+G4B_DEV u4 gload16_async(const void* sbase, uint32_t voff) {
+    u4 v;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
+    return v;
+}
+// Wait until at most N vector-memory operations are outstanding; the eight values are tied to the wait.
+template <int N>
+G4B_DEV void vm_wait8(u4 (&v)[8]) {
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+                 : "n"(N));
+}
+G4B_DEV void vm_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Wait until at most N LDS operations are outstanding; v is tied so its consumers stay behind the wait.
 template <int N>
 G4B_DEV void lds_wait(u4& v) {

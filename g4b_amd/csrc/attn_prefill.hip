@@ -7,54 +7,54 @@
 // without masks, edge tiles (sliding-window lower edge, causal diagonal, window end) compare
 // per element.
 //
-// Staging.  Tiles are double-buffered in LDS.  K goes global -> LDS directly
-// (global_load_lds_dwordx4, no registers): rows stay row-major and unpadded, the 16-byte pieces
-// of a row are XOR-swizzled with (row & 15) by choosing which global piece each lane fetches.
-// V passes through registers for an in-lane 8x8 16-bit transpose and is stored as V^T
-// ([d][key], 128-byte rows) with the 16-byte column groups XOR-swizzled.  Both are read back
-// with conflict-free ds_read_b128 directly in MFMA operand layout.
+// Staging.  K and V tiles are double-buffered in LDS and both travel global -> LDS directly
+// (global_load_lds_dwordx4: no registers, no LDS stores).  Rows stay row-major and unpadded; the
+// 16-byte pieces of a row are XOR-swizzled by choosing which global piece each lane fetches:
+// K with (row & 15), read back with ds_read_b128 as the A operand of S^T = K Q^T; V with
+// 4 * (row & 7) (whole 64-byte groups move), read back with ds_read_b64_tr_b16, which transposes
+// 4 keys x 16 columns inside each 16-lane group and so delivers V^T fragments without a transpose
+// pass.  Both read patterns are bank-conflict free.  The direct loads are issued a few at a time
+// between MFMA steps so the address unit never queues a burst.
 //
 // Math per tile and wave: S^T[64 keys x 32 rows] = K Q^T and O^T[D x 32 rows] += V^T P on
 // v_mfma_f32_32x32x16 (fp16 or bf16 operands, fp32 accumulate).  Q stays in registers as the B
 // operand; P never leaves registers: the accumulator layout of S^T is the B-operand layout of
 // the second product once the key order inside each 16-key group of V^T is permuted to match.
-// LDS operand reads run a fixed number of steps ahead of the MFMAs that consume them.
-// Softmax is online in fp32 with exp2 and scale*log2(e) folded into one FMA; the row statistics
-// live one row per lane pair (lane, lane^32).
+// The loop is software pipelined: S(kt+1) is computed while the softmax of S(kt) runs.  LDS
+// operand reads are volatile asm issued a fixed number of steps ahead of their MFMA and retired
+// with explicit lgkmcnt waits.  Softmax is online in fp32 with exp2 and scale*log2(e) folded into
+// one FMA; the row statistics live one row per lane pair (lane, lane^32); accumulators are
+// rescaled lazily.
 #include "common.hpp"
 #include "launch.hpp"
 
 namespace g4b {
 
-constexpr int PF_BM = 128;  // query rows per workgroup
-constexpr int PF_BN = 64;   // keys per tile
-constexpr int PF_PD = 4;    // LDS operand reads in flight ahead of the MFMA that uses them
+constexpr int PF_BM = 128;     // query rows per workgroup
+constexpr int PF_BN = 64;      // keys per tile
+constexpr int PF_PD = 4;       // LDS operand fetches in flight ahead of the MFMA that uses them
 constexpr float PF_TAU = 8.f;  // log2 of the growth of a row maximum that triggers a rescale
 
 template <int D>
 struct PfSmem {
-    static constexpr int KROW = D * 2;  // bytes per K row in LDS (unpadded, swizzled)
-    static constexpr int KBYTES = PF_BN * KROW;
-    static constexpr int VROW = PF_BN * 2;  // bytes per V^T row (64 keys), swizzled
-    static constexpr int VBYTES = D * VROW;
-    static constexpr int STAGE = KBYTES + VBYTES;
+    static constexpr int ROW = D * 2;  // bytes per K or V row, in memory and in LDS
+    static constexpr int TILE = PF_BN * ROW;
+    static constexpr int VSWZ = (D >= 256) ? 7 : 3;  // (V row & VSWZ) selects the 64-byte group swizzle
 };
-
-typedef __attribute__((address_space(1))) const void* gptr_t;
-typedef __attribute__((address_space(3))) void* lptr_t;
 
 template <int D, class T>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     using SM = PfSmem<D>;
     extern __shared__ __align__(16) char smem[];
-    constexpr int KSTEPS = D / 16;  // contraction steps of the first product
-    constexpr int DT = D / 32;      // 32-row tiles of O^T
-    constexpr int KCHUNKS = SM::KBYTES / 1024 / 4;  // 1 KiB direct-to-LDS loads per wave and tile
-    constexpr int ROWS_PER_CHUNK = 1024 / SM::KROW;
+    constexpr int KSTEPS = D / 16;               // contraction steps of the first product
+    constexpr int DT = D / 32;                   // 32-row tiles of O^T
+    constexpr int CHUNKS = SM::TILE / 1024 / 4;  // 1 KiB direct-to-LDS loads per wave and tile (K or V)
+    constexpr int ROWS_PER_CHUNK = 1024 / SM::ROW;
     constexpr int PIECES = D / 8;
-    constexpr int VSEG = D / 8;                 // 8-wide d segments per row
-    constexpr int VITEMS = (PF_BN / 8) * VSEG;  // (8-key group, d segment) items per tile
-    static_assert(VITEMS <= 256, "one V item per thread");
+    constexpr int QK_STEPS = 2 * KSTEPS;  // MFMAs of S^T = K Q^T per tile; step idx -> (c = idx/2, key tile mt = idx%2)
+    constexpr int PV_STEPS = 4 * DT;      // MFMAs of O^T += V^T P per tile; step idx -> (key group idx/DT, d tile idx%DT)
+    constexpr int N1 = 8;                 // QK steps issued next to the row-max part of the softmax
+    static_assert(PF_PD == 4, "the wait ladders are written for 4 fetches in flight");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     for (int i = 0; i < DT; ++i)
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;  // running max in log2 units (scaled), running sum (this lane's keys)
+    float m_run = -INFINITY, l_run = 0.f;  // exponent reference in log2 units (scaled), running sum (this lane's keys)
 
     if (hi_wg > lo_wg) {
         // Q as B operand: lane (row n32, half h2), step c: d = 16c + 8*h2 .. +8
@@ -103,34 +103,32 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 
         const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
         const char* vbase = static_cast<const char*>(p.v) + ((int64_t)b * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
-        auto key_off = [&](int j) -> uint32_t {
+        auto key_off = [&](int j) -> uint32_t {  // byte offset of logical key j (clamped to the window) in the ring
             j = min(max(j, 0), si.window - 1);
             int r = si.ring_start + j;
             r = (r >= KV_CTX) ? r - KV_CTX : r;
-            return (uint32_t)r * (uint32_t)(D * 2);
+            return (uint32_t)r * (uint32_t)SM::ROW;
         };
 
-        // ---- staging roles ------------------------------------------------------------------------
-        // K: wave `wave` issues KCHUNKS direct loads; chunk c covers LDS bytes [c*1024, +1024) of the K tile.
-        const int k_row_in_chunk = lane / PIECES;  // 0 .. ROWS_PER_CHUNK-1
-        const int k_piece_lds = lane % PIECES;
-        // V: thread item = (8-key group q8, d segment)
-        const int v_q8 = tid / VSEG, v_dseg = tid % VSEG;
-        const bool v_item = (VITEMS == 256) || tid < VITEMS;
-        u4 vst[8];
-
+        // ---- staging ------------------------------------------------------------------------------------------
+        // LDS map: K stages at [0, 2*TILE), V stages at [2*TILE, 4*TILE).  Wave `wave` moves chunks
+        // wave*CHUNKS .. +CHUNKS of each tile; chunk c covers bytes [c*1024, +1024) of the tile, lane l its piece l.
+        const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the dynamic segment
+        const int st_row_in_chunk = lane / PIECES;        // 0 .. ROWS_PER_CHUNK-1
+        const int st_piece_lds = lane % PIECES;           // 16-byte piece position inside the LDS row
+        auto st_row = [&](int i) { return (wave * CHUNKS + i) * ROWS_PER_CHUNK + st_row_in_chunk; };
+        auto k_piece = [&](int row) { return st_piece_lds ^ (row & 15); };
+        auto v_piece = [&](int row) { return st_piece_lds ^ (4 * (row & SM::VSWZ)); };
         // A tile is "plain" when its 64 keys lie inside the window and do not straddle the ring seam: then its rows
         // are consecutive in memory and every lane's source offset is a loop constant added to one scalar base.
         // Only the first / last tiles of a slot and the one on the seam take the general path with per-row clamping.
-        uint32_t k_const[KCHUNKS], v_const[8];
+        uint32_t k_const[CHUNKS], v_const[CHUNKS];
 #pragma unroll
-        for (int i = 0; i < KCHUNKS; ++i) {
-            const int row = (wave * KCHUNKS + i) * ROWS_PER_CHUNK + k_row_in_chunk;
-            k_const[i] = (uint32_t)row * SM::KROW + (uint32_t)(k_piece_lds ^ (row & 15)) * 16u;
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int row = st_row(i);
+            k_const[i] = (uint32_t)row * SM::ROW + (uint32_t)k_piece(row) * 16u;
+            v_const[i] = (uint32_t)row * SM::ROW + (uint32_t)v_piece(row) * 16u;
         }
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            v_const[j] = (uint32_t)((v_q8 >> 1) * 16 + (v_q8 & 1) * 4 + 8 * (j >> 2) + (j & 3)) * SM::KROW + (uint32_t)v_dseg * 16u;
         auto plain_row0 = [&](int kt) -> int {  // ring row of the tile's first key, or -1
             const int jb = kt * PF_BN;
             if (jb + PF_BN > si.window) return -1;
@@ -138,105 +136,89 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             r0 = (r0 >= KV_CTX) ? r0 - KV_CTX : r0;
             return (r0 + PF_BN <= KV_CTX) ? r0 : -1;
         };
-        auto issue_k = [&](int kt, int stage) {
-            const int jb = kt * PF_BN;
-            char* ks = smem + stage * SM::KBYTES;
+        // Source of K or V tile kt as scalar base + per-lane byte offsets.
+        auto tile_src = [&](int kt, bool is_v, const char*& src, uint32_t(&ofs)[CHUNKS]) {
             const int r0 = plain_row0(kt);
+            const char* base = is_v ? vbase : kbase;
             if (r0 >= 0) {
-                const char* tb = kbase + (int64_t)r0 * SM::KROW;
+                src = base + (int64_t)r0 * SM::ROW;
 #pragma unroll
-                for (int i = 0; i < KCHUNKS; ++i)
-                    __builtin_amdgcn_global_load_lds((gptr_t)(tb + k_const[i]), (lptr_t)(ks + (wave * KCHUNKS + i) * 1024), 16, 0, 0);
+                for (int i = 0; i < CHUNKS; ++i) ofs[i] = is_v ? v_const[i] : k_const[i];
             } else {
+                src = base;
 #pragma unroll
-                for (int i = 0; i < KCHUNKS; ++i) {
-                    const int chunk = wave * KCHUNKS + i;
-                    const int row = chunk * ROWS_PER_CHUNK + k_row_in_chunk;
-                    const int piece = k_piece_lds ^ (row & 15);
-                    const char* src = kbase + key_off(jb + row) + (uint32_t)piece * 16u;
-                    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ks + chunk * 1024), 16, 0, 0);
+                for (int i = 0; i < CHUNKS; ++i) {
+                    const int row = st_row(i);
+                    ofs[i] = key_off(kt * PF_BN + row) + (uint32_t)(is_v ? v_piece(row) : k_piece(row)) * 16u;
                 }
             }
         };
-        auto issue_v = [&](int kt) {
-            const int jb = kt * PF_BN;
-            const int r0 = plain_row0(kt);
-            if (r0 >= 0) {
-                const char* tb = vbase + (int64_t)r0 * SM::KROW;
-                if (v_item) {
+        const uint32_t wave_chunk0 = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (CHUNKS * 1024);
+        auto stage_whole_tile = [&](int kt, bool is_v, int stage) {  // prologue only: all chunks at once
+            const char* src;
+            uint32_t ofs[CHUNKS];
+            tile_src(kt, is_v, src, ofs);
+            const uint32_t dst = lds0 + (is_v ? 2 * SM::TILE : 0) + stage * SM::TILE + wave_chunk0;
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) vst[j] = ld16(tb, v_const[j]);
-                }
-            } else {
-                // 8-key group q8: 16-key group q8/2, half q8 & 1; slot j -> key 8*(j/4) + 4*half + j%4
-                const int kb16 = jb + (v_q8 >> 1) * 16 + (v_q8 & 1) * 4;
-                if (v_item) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        vst[j] = ld16(vbase, key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)v_dseg * 16u);
-                }
-            }
-        };
-        auto store_v = [&](int stage) {
-            char* vs = smem + 2 * SM::KBYTES + stage * SM::VBYTES;
-            if (v_item) {
-                u4 vt[8];
-                transpose8x8_b16(vst, vt);
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj) {
-                    const int d = v_dseg * 8 + jj;
-                    const int slot = v_q8 ^ ((jj ^ v_dseg) & 7);
-                    *reinterpret_cast<u4*>(vs + d * SM::VROW + slot * 16) = vt[jj];
-                }
-            }
+            for (int i = 0; i < CHUNKS; ++i) dma16_to_lds(src, ofs[i], dst + i * 1024);
         };
 
-        // ---- operand read offsets ------------------------------------------------------------------
-        // LDS map: K stages at [0, 2*KBYTES), V^T stages at [2*KBYTES, 2*KBYTES + 2*VBYTES).
+        // ---- operand read offsets (bytes from the start of a stage pair) ----------------------------------------
         // K^T step (mt, c): row mt*32 + n32, piece 2c + h2, swizzled with (row & 15) = (n32 & 15)
         uint32_t koff[8];
 #pragma unroll
-        for (int c8 = 0; c8 < 8; ++c8) koff[c8] = (uint32_t)n32 * SM::KROW + (uint32_t)(((2 * c8 + h2) ^ (n32 & 15)) * 16);
-        // V^T step (dt, mt, u): row d = 32*dt + n32, column group (4*mt + 2*u + h2) ^ swz(d)
-        uint32_t voff[2][4];
+        for (int c8 = 0; c8 < 8; ++c8) koff[c8] = (uint32_t)n32 * SM::ROW + (uint32_t)(((2 * c8 + h2) ^ (n32 & 15)) * 16);
+        // V^T fragment of step (cu, dt): d = 32dt + n32, keys {16cu + 4h2 + 0..3, 16cu + 8 + 4h2 + 0..3} (the order in
+        // which this lane half holds P), fetched with two transposing reads.  Inside a 16-lane group, lane 4r + q
+        // points at columns 4q..4q+3 of key r of the block and receives the group's column (lane % 16) of 4 keys.
+        const int tr_r = (lane & 15) >> 2, tr_q = lane & 3, tr_dhalf = (lane >> 4) & 1;
+        const int tr_key = 4 * h2 + tr_r;  // key (mod 16) this lane points at
+        uint32_t voff[DT];
 #pragma unroll
-        for (int par = 0; par < 2; ++par) {
-            const int d = par * 32 + n32;
-            const int sw = (d ^ (d >> 3)) & 7;
-#pragma unroll
-            for (int cu = 0; cu < 4; ++cu) voff[par][cu] = 2 * SM::KBYTES + (uint32_t)n32 * SM::VROW + (uint32_t)(((2 * cu + h2) ^ sw) * 16);
+        for (int dt = 0; dt < DT; ++dt) {
+            const int piece = dt * 4 + tr_dhalf * 2 + (tr_q >> 1);
+            voff[dt] = 2 * SM::TILE + (uint32_t)tr_key * SM::ROW + (uint32_t)((piece ^ (4 * (tr_key & SM::VSWZ))) * 16) +
+                       (uint32_t)(tr_q & 1) * 8u;
         }
-        constexpr int QK_STEPS = 2 * KSTEPS;  // MFMAs of S^T = K Q^T per tile; step idx -> (c = idx/2, key tile mt = idx%2)
-        constexpr int PV_STEPS = 4 * DT;      // MFMAs of O^T += V^T P per tile; step idx -> (key group idx/DT, d tile idx%DT)
-        const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the dynamic segment
         // Operand reads are issued as volatile asm, PF_PD steps ahead of the MFMA that consumes them, and
         // retired with explicit lgkmcnt waits: LDS returns data in order, so "at most n outstanding" is exact
         // for the oldest read whatever else the compiler has in flight.
-        uint32_t kaddr[8], vaddr[2][4];
-        // `left` = reads of the same sequence issued after the one being retired (a constant after unrolling)
+        uint32_t kaddr[8], vaddr[DT];
+        auto k_issue = [&](int idx) -> u4 {  // needs kaddr[] of the stage
+            const int c = idx >> 1, mt = idx & 1;
+            return lds_read16(kaddr[c & 7], mt * 32 * SM::ROW + (c >> 3) * 256);
+        };
+        struct VFrag {
+            u2 lo, hi;
+        };
+        auto v_issue = [&](int idx) -> VFrag {  // needs vaddr[] of the stage
+            const int cu = idx / DT, dt = idx % DT;
+            VFrag f;
+            f.lo = lds_read8_tr16(vaddr[dt], cu * 16 * SM::ROW);
+            f.hi = lds_read8_tr16(vaddr[dt], (cu * 16 + 8) * SM::ROW);
+            return f;
+        };
+        // `left` = fetches of the same sequence issued after the one being retired (a constant after unrolling)
         auto wait_left = [&](u4& a, int left) {
-            static_assert(PF_PD == 4, "wait ladder below is written for 4 reads in flight");
             if (left >= 3) lds_wait<3>(a);
             else if (left == 2) lds_wait<2>(a);
             else if (left == 1) lds_wait<1>(a);
             else lds_wait<0>(a);
         };
-        auto k_issue = [&](int idx) -> u4 {  // needs kaddr[] of the stage
-            const int c = idx >> 1, mt = idx & 1;
-            return lds_read16(kaddr[c & 7], mt * 32 * SM::KROW + (c >> 3) * 256);
-        };
-        auto v_issue = [&](int idx) -> u4 {
-            const int cu = idx / DT, dt = idx % DT;
-            return lds_read16(vaddr[dt & 1][cu], dt * 32 * SM::VROW);
+        auto wait_left2 = [&](VFrag& f, int left) {  // every fragment is two reads
+            if (left >= 3) lds_wait2<6>(f.lo, f.hi);
+            else if (left == 2) lds_wait2<4>(f.lo, f.hi);
+            else if (left == 1) lds_wait2<2>(f.lo, f.hi);
+            else lds_wait2<0>(f.lo, f.hi);
         };
 
         const int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
 
         // ---- prologue: K(kt0), K(kt0+1), V(kt0) staged; S(kt0) computed --------------------------------
-        issue_k(kt0, 0);
-        issue_k(kt0 + 1, 1);
-        issue_v(kt0);
-        store_v(0);
+        stage_whole_tile(kt0, false, 0);
+        stage_whole_tile(kt0 + 1, false, 1);
+        stage_whole_tile(kt0, true, 0);
+        vm_wait_all();
         __syncthreads();
         f16v s_cur[2];
 #pragma unroll
@@ -262,50 +244,24 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 
         // One tile: softmax of S(kt) and O += V(kt) P, overlapped with S(kt+1) = K(kt+1) Q^T.
         // par = (kt - kt0) & 1: V(kt) sits in V stage par, K(kt+1) in K stage par^1; K(kt+2) is fetched into K
-        // stage par and V(kt+1) into V stage par^1 while this tile computes.
+        // stage par and V(kt+1) into V stage par^1 while this tile computes.  The tiles after the last one are
+        // fetched (addresses are clamped to the window) and multiplied too; nobody reads the results.
         for (int kt = kt0; kt <= kt1; ++kt) {
-            constexpr int N1 = 8;  // QK steps issued next to the row-max part of the softmax
             const int par = (kt - kt0) & 1;
-            // the tiles after the last one are fetched (addresses are clamped to the window) and multiplied too;
-            // nobody reads the results
-            // Sources of K(kt+2) and V(kt+1): scalar base + per-lane offset (loop constants on plain tiles).  The
-            // loads themselves are issued a few at a time between the MFMA steps below so that the address unit is
-            // never handed more than one instruction per wave at once.
-            const char* ksrc = kbase;
-            const char* vsrc = vbase;
-            uint32_t kofs[KCHUNKS], vofs[8];
+            // Sources of K(kt+2) and V(kt+1).  The loads themselves are issued a few at a time between the MFMA
+            // steps below so that the address unit is never handed more than one instruction per wave at once.
+            const char *ksrc, *vsrc;
+            uint32_t kofs[CHUNKS], vofs[CHUNKS];
+            tile_src(kt + 2, false, ksrc, kofs);
+            tile_src(kt + 1, true, vsrc, vofs);
+            const uint32_t kdst = lds0 + par * SM::TILE + wave_chunk0;
+            const uint32_t vdst = lds0 + 2 * SM::TILE + (par ^ 1) * SM::TILE + wave_chunk0;
             {
-                const int rk = plain_row0(kt + 2), rv = plain_row0(kt + 1);
-                if (rk >= 0) {
-                    ksrc = kbase + (int64_t)rk * SM::KROW;
-#pragma unroll
-                    for (int i = 0; i < KCHUNKS; ++i) kofs[i] = k_const[i];
-                } else {
-#pragma unroll
-                    for (int i = 0; i < KCHUNKS; ++i) {
-                        const int row = (wave * KCHUNKS + i) * ROWS_PER_CHUNK + k_row_in_chunk;
-                        kofs[i] = key_off((kt + 2) * PF_BN + row) + (uint32_t)(k_piece_lds ^ (row & 15)) * 16u;
-                    }
-                }
-                if (rv >= 0) {
-                    vsrc = vbase + (int64_t)rv * SM::KROW;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) vofs[j] = v_const[j];
-                } else {
-                    const int kb16 = (kt + 1) * PF_BN + (v_q8 >> 1) * 16 + (v_q8 & 1) * 4;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) vofs[j] = key_off(kb16 + 8 * (j >> 2) + (j & 3)) + (uint32_t)v_dseg * 16u;
-                }
-            }
-            const uint32_t kdst = lds0 + par * SM::KBYTES + (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (KCHUNKS * 1024);
-            {
-                const uint32_t kb = lds0 + (par ^ 1) * SM::KBYTES, vb = lds0 + par * SM::VBYTES;
+                const uint32_t kb = lds0 + (par ^ 1) * SM::TILE, vb = lds0 + par * SM::TILE;
 #pragma unroll
                 for (int c8 = 0; c8 < 8; ++c8) kaddr[c8] = kb + koff[c8];
 #pragma unroll
-                for (int q = 0; q < 2; ++q)
-#pragma unroll
-                    for (int cu = 0; cu < 4; ++cu) vaddr[q][cu] = vb + voff[q][cu];  // voff includes the 2*KBYTES base
+                for (int dt = 0; dt < DT; ++dt) vaddr[dt] = vb + voff[dt];  // voff includes the 2*TILE base
             }
 
             // ---- edge tiles only: mask S(kt) before anything else so the rest of the tile is one straight block
@@ -334,11 +290,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                 wait_left(a, QK_STEPS - 1 - idx);
                 if (idx + PF_PD < QK_STEPS) abuf[idx % PF_PD] = k_issue(idx + PF_PD);
                 s_nxt[idx & 1] = T::mfma32(a, qf[idx >> 1], s_nxt[idx & 1]);
-                // one of the eight V(kt+1) row loads every few steps of the second part
-                constexpr int VSTRIDE = (QK_STEPS - N1) / 8;
-                if (idx >= N1 && (idx - N1) % VSTRIDE == 0 && (idx - N1) / VSTRIDE < 8) {
-                    if (v_item) vst[(idx - N1) / VSTRIDE] = gload16_async(vsrc, vofs[(idx - N1) / VSTRIDE]);
-                }
+                // one of the V(kt+1) direct loads every few steps of the second part
+                constexpr int VSTRIDE = (QK_STEPS - N1) / CHUNKS;
+                if (idx >= N1 && (idx - N1) % VSTRIDE == 0 && (idx - N1) / VSTRIDE < CHUNKS)
+                    dma16_to_lds(vsrc, vofs[(idx - N1) / VSTRIDE], vdst + ((idx - N1) / VSTRIDE) * 1024);
             };
 #pragma unroll
             for (int idx = 0; idx < N1; ++idx) qk_step(idx);
@@ -389,7 +344,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                         psum += e[j];
                     }
                     pf[mt][u] = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
-                    // six of the remaining K Q^T steps next to each quarter of the exponentials
+                    // a quarter of the remaining K Q^T steps next to each quarter of the exponentials
 #pragma unroll
                     for (int q = 0; q < (QK_STEPS - N1) / 4; ++q) qk_step(N1 + (mt * 2 + u) * ((QK_STEPS - N1) / 4) + q);
                 }
@@ -397,22 +352,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 
             // ---- O^T += V^T P : (key group) outer, d tile inner -> consecutive MFMAs are independent ----------
             {
-                u4 vbuf[PF_PD];
+                VFrag vbuf[PF_PD];
 #pragma unroll
                 for (int i = 0; i < PF_PD; ++i) vbuf[i] = v_issue(i);
 #pragma unroll
                 for (int idx = 0; idx < PV_STEPS; ++idx) {
-                    u4 a = vbuf[idx % PF_PD];
-                    wait_left(a, PV_STEPS - 1 - idx);
+                    VFrag f = vbuf[idx % PF_PD];
+                    wait_left2(f, PV_STEPS - 1 - idx);
                     if (idx + PF_PD < PV_STEPS) vbuf[idx % PF_PD] = v_issue(idx + PF_PD);
                     const int cu = idx / DT, dt = idx % DT;
+                    const u4 a = {f.lo[0], f.lo[1], f.hi[0], f.hi[1]};
                     acc[dt] = T::mfma32(a, pf[cu >> 1][cu & 1], acc[dt]);
-                    // one of the K(kt+2) direct-to-LDS loads every other step of the first half
-                    if (idx % 2 == 0 && idx / 2 < KCHUNKS) dma16_to_lds(ksrc, kofs[idx / 2], kdst + (idx / 2) * 1024);
+                    // one of the K(kt+2) direct loads every other step of the first half
+                    if (idx % 2 == 0 && idx / 2 < CHUNKS) dma16_to_lds(ksrc, kofs[idx / 2], kdst + (idx / 2) * 1024);
                 }
             }
-            vm_wait8<KCHUNKS>(vst);  // the V loads were issued before the K loads
-            store_v(par ^ 1);
             vm_wait_all();
             __syncthreads();
             s_cur[0] = s_nxt[0];
@@ -421,7 +375,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     }
 
     // ---- epilogue: lane (row n32, half h2) holds d = 32*dt + 8*(i/4) + 4*h2 + i%4 -----------------
-    float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float l_tot = half_swap_sum(l_run);
     if (row_ok) {
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
 #pragma unroll
@@ -438,7 +392,7 @@ template <int D, class T>
 static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     const int TOKB = PF_BM / p.R;
     dim3 grid((p.Tq + TOKB - 1) / TOKB, p.G, p.B);
-    const int smem = 2 * PfSmem<D>::STAGE;
+    const int smem = 4 * PfSmem<D>::TILE;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T>),

@@ -186,6 +186,20 @@ G4B_DEV void lds_wait(u4& v) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
 }
 
+// Transposing 8-byte LDS read of 16-bit elements (issued where it is written, retire with lds_wait2<n>).
+// Inside every group of 16 lanes, lane s supplies the address of 4 consecutive elements E[s][0..3]; lane i receives
+// E[i/4][i%4], E[4 + i/4][i%4], E[8 + i/4][i%4], E[12 + i/4][i%4].  With lane 4r+q pointing at columns 4q..4q+3 of row r
+// of a 4 x 16 block, lane i receives column i of the four rows.
+G4B_DEV u2 lds_read8_tr16(uint32_t lds_addr, int imm) {
+    u2 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(imm));
+    return v;
+}
+template <int N>
+G4B_DEV void lds_wait2(u2& a, u2& b) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
 // In-lane 8x8 transpose of 16-bit elements.  in[s] holds elements (s, 0..7); out[j] holds (0..7, j).
 G4B_DEV void transpose8x8_b16(const u4 (&in)[8], u4 (&out)[8]) {
 #pragma unroll

@@ -32,7 +32,7 @@ namespace g4b {
 
 constexpr int PF_BM = 128;     // query rows per workgroup
 constexpr int PF_BN = 64;      // keys per tile
-constexpr int PF_PD = 4;       // LDS operand fetches in flight ahead of the MFMA that uses them
+constexpr int PF_PD = 6;       // LDS operand fetches in flight (issued and retired in pairs)
 constexpr float PF_TAU = 8.f;  // log2 of the growth of a row maximum that triggers a rescale
 
 template <int D>
@@ -41,6 +41,25 @@ struct PfSmem {
     static constexpr int TILE = PF_BN * ROW;
     static constexpr int VSWZ = (D >= 256) ? 7 : 3;  // (V row & VSWZ) selects the 64-byte group swizzle
 };
+
+// Linear workgroup id -> (head, query tile rank) bookkeeping shared by the kernel and its launcher.
+struct PfMap {
+    int heads, nq, mode, grid;
+};
+__host__ __device__ inline PfMap pf_map(int heads, int nq) {
+    PfMap m;
+    m.heads = heads;
+    m.nq = nq;
+    if (heads <= 8 && 8 % heads == 0) {
+        const int share = 8 / heads;
+        m.mode = 1;
+        m.grid = 8 * ((nq + share - 1) / share);
+    } else {
+        m.mode = (heads % 8 == 0) ? 2 : 0;
+        m.grid = heads * nq;
+    }
+    return m;
+}
 
 template <int D, class T>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
@@ -54,15 +73,35 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     constexpr int QK_STEPS = 2 * KSTEPS;  // MFMAs of S^T = K Q^T per tile; step idx -> (c = idx/2, key tile mt = idx%2)
     constexpr int PV_STEPS = 4 * DT;      // MFMAs of O^T += V^T P per tile; step idx -> (key group idx/DT, d tile idx%DT)
     constexpr int N1 = 8;                 // QK steps issued next to the row-max part of the softmax
-    static_assert(PF_PD == 4, "the wait ladders are written for 4 fetches in flight");
+    static_assert(PF_PD == 6, "the wait ladders are written for three pairs of fetches in flight");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int n32 = lane & 31, h2 = lane >> 5;
     const int R = p.R, Tq = p.Tq, KV_CTX = p.KV_CTX;
     const int TOKB = PF_BM / R;
-    const int qtile = (int)gridDim.x - 1 - (int)blockIdx.x;  // heaviest (latest) tiles first
-    const int g = blockIdx.y, b = blockIdx.z;
+    // Work item of this workgroup: (kv head of a slot, query tile).  Workgroups are handed to the 8 XCDs round-robin
+    // by their linear id and every XCD has an L2 of its own, so the ids are mapped such that an XCD walks the K/V of
+    // as few heads as possible, its workgroups start at the same key and advance together (one fetch from memory
+    // serves the XCD), the heaviest (latest) query tiles start first, and the XCDs get equal shares.
+    const PfMap map = pf_map(p.G * p.B, (Tq + TOKB - 1) / TOKB);
+    int head, rank;
+    {
+        const int f = blockIdx.x, x = f & 7, j = f >> 3;
+        if (map.mode == 1) {  // heads divide 8: 8 / heads XCDs share a head and take its query tiles in turn
+            head = x % map.heads;
+            rank = j * (8 / map.heads) + x / map.heads;
+        } else if (map.mode == 2) {  // 8 divides heads: every XCD owns heads / 8 heads
+            head = (j % (map.heads / 8)) * 8 + x;
+            rank = j / (map.heads / 8);
+        } else {
+            head = f % map.heads;
+            rank = f / map.heads;
+        }
+    }
+    if (rank >= map.nq) return;
+    const int qtile = map.nq - 1 - rank;
+    const int g = head % p.G, b = head / p.G;
 
     const SlotInfo si = slot_info(p, b);
     if (!si.active) return;
@@ -198,18 +237,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             f.hi = lds_read8_tr16(vaddr[dt], (cu * 16 + 8) * SM::ROW);
             return f;
         };
-        // `left` = fetches of the same sequence issued after the one being retired (a constant after unrolling)
-        auto wait_left = [&](u4& a, int left) {
-            if (left >= 3) lds_wait<3>(a);
-            else if (left == 2) lds_wait<2>(a);
-            else if (left == 1) lds_wait<1>(a);
-            else lds_wait<0>(a);
+        // Reads are retired a pair at a time; `left` = pairs of the same sequence issued after the one being retired
+        // (a constant after unrolling).
+        auto wait_pair = [&](u4& a0, u4& a1, int left) {
+            if (left >= 2) lds_wait_pair<4>(a0, a1);
+            else if (left == 1) lds_wait_pair<2>(a0, a1);
+            else lds_wait_pair<0>(a0, a1);
         };
-        auto wait_left2 = [&](VFrag& f, int left) {  // every fragment is two reads
-            if (left >= 3) lds_wait2<6>(f.lo, f.hi);
-            else if (left == 2) lds_wait2<4>(f.lo, f.hi);
-            else if (left == 1) lds_wait2<2>(f.lo, f.hi);
-            else lds_wait2<0>(f.lo, f.hi);
+        auto wait_pair2 = [&](VFrag& f0, VFrag& f1, int left) {  // every fragment is two reads
+            if (left >= 2) lds_wait4<8>(f0.lo, f0.hi, f1.lo, f1.hi);
+            else if (left == 1) lds_wait4<4>(f0.lo, f0.hi, f1.lo, f1.hi);
+            else lds_wait4<0>(f0.lo, f0.hi, f1.lo, f1.hi);
         };
 
         const int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
@@ -233,11 +271,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 #pragma unroll
             for (int i = 0; i < PF_PD; ++i) abuf[i] = k_issue(i);
 #pragma unroll
-            for (int idx = 0; idx < QK_STEPS; ++idx) {
-                u4 a = abuf[idx % PF_PD];
-                wait_left(a, QK_STEPS - 1 - idx);
-                if (idx + PF_PD < QK_STEPS) abuf[idx % PF_PD] = k_issue(idx + PF_PD);
-                s_cur[idx & 1] = T::mfma32(a, qf[idx >> 1], s_cur[idx & 1]);
+            for (int idx = 0; idx < QK_STEPS; idx += 2) {
+                u4 a0 = abuf[idx % PF_PD], a1 = abuf[(idx + 1) % PF_PD];
+                wait_pair(a0, a1, (QK_STEPS - 2 - idx) / 2);
+                if (idx + PF_PD < QK_STEPS) {
+                    abuf[idx % PF_PD] = k_issue(idx + PF_PD);
+                    abuf[(idx + 1) % PF_PD] = k_issue(idx + 1 + PF_PD);
+                }
+                s_cur[0] = T::mfma32(a0, qf[idx >> 1], s_cur[0]);
+                s_cur[1] = T::mfma32(a1, qf[idx >> 1], s_cur[1]);
             }
         }
         __syncthreads();  // every wave is done with K stage 0 before the loop refills it
@@ -277,26 +319,32 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             }
 
             f16v s_nxt[2];
-            u4 abuf[PF_PD];
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 s_nxt[0][j] = 0.f;
                 s_nxt[1][j] = 0.f;
             }
+            u4 abuf[PF_PD];
 #pragma unroll
             for (int i = 0; i < PF_PD; ++i) abuf[i] = k_issue(i);
-            auto qk_step = [&](int idx) {
-                u4 a = abuf[idx % PF_PD];
-                wait_left(a, QK_STEPS - 1 - idx);
-                if (idx + PF_PD < QK_STEPS) abuf[idx % PF_PD] = k_issue(idx + PF_PD);
-                s_nxt[idx & 1] = T::mfma32(a, qf[idx >> 1], s_nxt[idx & 1]);
-                // one of the V(kt+1) direct loads every few steps of the second part
-                constexpr int VSTRIDE = (QK_STEPS - N1) / CHUNKS;
-                if (idx >= N1 && (idx - N1) % VSTRIDE == 0 && (idx - N1) / VSTRIDE < CHUNKS)
-                    dma16_to_lds(vsrc, vofs[(idx - N1) / VSTRIDE], vdst + ((idx - N1) / VSTRIDE) * 1024);
+            auto qk_pair = [&](int idx) {  // steps idx (key tile 0) and idx + 1 (key tile 1) of contraction step idx / 2
+                u4 a0 = abuf[idx % PF_PD], a1 = abuf[(idx + 1) % PF_PD];
+                wait_pair(a0, a1, (QK_STEPS - 2 - idx) / 2);
+                if (idx + PF_PD < QK_STEPS) {
+                    abuf[idx % PF_PD] = k_issue(idx + PF_PD);
+                    abuf[(idx + 1) % PF_PD] = k_issue(idx + 1 + PF_PD);
+                }
+                s_nxt[0] = T::mfma32(a0, qf[idx >> 1], s_nxt[0]);
+                s_nxt[1] = T::mfma32(a1, qf[idx >> 1], s_nxt[1]);
+                // One direct load per pair: K(kt+2) first (its stage was released by the barrier that ended the
+                // previous tile and it is needed first), then V(kt+1).  Issued this early, the loads have the rest
+                // of the tile to land before the closing barrier waits for them.
+                if (idx / 2 < CHUNKS) dma16_to_lds(ksrc, kofs[idx / 2], kdst + (idx / 2) * 1024);
+                if (idx / 2 >= CHUNKS && idx / 2 < 2 * CHUNKS)
+                    dma16_to_lds(vsrc, vofs[idx / 2 - CHUNKS], vdst + (idx / 2 - CHUNKS) * 1024);
             };
 #pragma unroll
-            for (int idx = 0; idx < N1; ++idx) qk_step(idx);
+            for (int idx = 0; idx < N1; idx += 2) qk_pair(idx);
 
             // ---- softmax, part 1: row maximum --------------------------------------------------------------
             float mx = fmaxf(s_cur[0][0], s_cur[1][0]);
@@ -339,14 +387,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                 for (int u = 0; u < 2; ++u) {
                     float e[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        e[j] = fast_exp2(__builtin_fmaf(s_cur[mt][8 * u + j], p.c, -m_safe));
-                        psum += e[j];
-                    }
+                    for (int j = 0; j < 8; ++j) e[j] = fast_exp2(__builtin_fmaf(s_cur[mt][8 * u + j], p.c, -m_safe));
                     pf[mt][u] = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
+                    // the row sum adds up the rounded values the second product uses
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t w = pf[mt][u][j];
+                        psum = T::sum2(w, psum);
+                    }
                     // a quarter of the remaining K Q^T steps next to each quarter of the exponentials
 #pragma unroll
-                    for (int q = 0; q < (QK_STEPS - N1) / 4; ++q) qk_step(N1 + (mt * 2 + u) * ((QK_STEPS - N1) / 4) + q);
+                    for (int q = 0; q < (QK_STEPS - N1) / 4; q += 2) qk_pair(N1 + (mt * 2 + u) * ((QK_STEPS - N1) / 4) + q);
                 }
             l_run += psum;
 
@@ -356,15 +407,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 #pragma unroll
                 for (int i = 0; i < PF_PD; ++i) vbuf[i] = v_issue(i);
 #pragma unroll
-                for (int idx = 0; idx < PV_STEPS; ++idx) {
-                    VFrag f = vbuf[idx % PF_PD];
-                    wait_left2(f, PV_STEPS - 1 - idx);
-                    if (idx + PF_PD < PV_STEPS) vbuf[idx % PF_PD] = v_issue(idx + PF_PD);
-                    const int cu = idx / DT, dt = idx % DT;
-                    const u4 a = {f.lo[0], f.lo[1], f.hi[0], f.hi[1]};
-                    acc[dt] = T::mfma32(a, pf[cu >> 1][cu & 1], acc[dt]);
-                    // one of the K(kt+2) direct loads every other step of the first half
-                    if (idx % 2 == 0 && idx / 2 < CHUNKS) dma16_to_lds(ksrc, kofs[idx / 2], kdst + (idx / 2) * 1024);
+                for (int idx = 0; idx < PV_STEPS; idx += 2) {
+                    VFrag f0 = vbuf[idx % PF_PD], f1 = vbuf[(idx + 1) % PF_PD];
+                    wait_pair2(f0, f1, (PV_STEPS - 2 - idx) / 2);
+                    if (idx + PF_PD < PV_STEPS) {
+                        vbuf[idx % PF_PD] = v_issue(idx + PF_PD);
+                        vbuf[(idx + 1) % PF_PD] = v_issue(idx + 1 + PF_PD);
+                    }
+                    const int cu = idx / DT, dt = idx % DT;  // DT is even: both steps share the key group
+                    const u4 a0 = {f0.lo[0], f0.lo[1], f0.hi[0], f0.hi[1]};
+                    const u4 a1 = {f1.lo[0], f1.lo[1], f1.hi[0], f1.hi[1]};
+                    acc[dt] = T::mfma32(a0, pf[cu >> 1][cu & 1], acc[dt]);
+                    acc[dt + 1] = T::mfma32(a1, pf[cu >> 1][cu & 1], acc[dt + 1]);
                 }
             }
             vm_wait_all();
@@ -391,7 +445,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 template <int D, class T>
 static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     const int TOKB = PF_BM / p.R;
-    dim3 grid((p.Tq + TOKB - 1) / TOKB, p.G, p.B);
+    dim3 grid(pf_map(p.G * p.B, (p.Tq + TOKB - 1) / TOKB).grid);
     const int smem = 4 * PfSmem<D>::TILE;
     static bool attr_set = false;
     if (!attr_set) {

@@ -33,6 +33,12 @@ struct F16 {
         h2 v = {(_Float16)lo, (_Float16)hi};
         return __builtin_bit_cast(uint32_t, v);
     }
+    // acc + both halves of a packed pair, accumulated in fp32 (v_dot2_f32_f16 against (1, 1))
+    static G4B_DEV float sum2(uint32_t w, float acc) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w), ones, acc, false);
+    }
     static G4B_DEV float lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); }
     static G4B_DEV float hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
 };
@@ -50,6 +56,7 @@ struct BF16 {
         b2 v = {(__bf16)lo, (__bf16)hi};
         return __builtin_bit_cast(uint32_t, v);
     }
+    static G4B_DEV float sum2(uint32_t w, float acc) { return acc + lo(w) + hi(w); }
     static G4B_DEV float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
     static G4B_DEV float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 };
@@ -154,7 +161,7 @@ G4B_DEV float half_swap_sum(float x) {
     return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
 }
 
-// 16-byte LDS read issued where it is written (volatile asm), to be retired by lds_wait<n> on the same value.
+// 16-byte LDS read issued where it is written (volatile asm), to be retired by lds_wait_pair<n> on the same value.
 G4B_DEV u4 lds_read16(uint32_t lds_addr, int imm) {
     u4 v;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(imm));
@@ -165,28 +172,9 @@ G4B_DEV u4 lds_read16(uint32_t lds_addr, int imm) {
 G4B_DEV void dma16_to_lds(const void* sbase, uint32_t voff, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
 }
-// 16-byte global load issued where it is written; retire with vm_wait8 before the values are used.
-G4B_DEV u4 gload16_async(const void* sbase, uint32_t voff) {
-    u4 v;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
-    return v;
-}
-// Wait until at most N vector-memory operations are outstanding; the eight values are tied to the wait.
-template <int N>
-G4B_DEV void vm_wait8(u4 (&v)[8]) {
-    asm volatile("s_waitcnt vmcnt(%8)"
-                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
-                 : "n"(N));
-}
 G4B_DEV void vm_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-// Wait until at most N LDS operations are outstanding; v is tied so its consumers stay behind the wait.
-template <int N>
-G4B_DEV void lds_wait(u4& v) {
-    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
-}
-
-// Transposing 8-byte LDS read of 16-bit elements (issued where it is written, retire with lds_wait2<n>).
+// Transposing 8-byte LDS read of 16-bit elements (issued where it is written, retire with lds_wait4<n>).
 // Inside every group of 16 lanes, lane s supplies the address of 4 consecutive elements E[s][0..3]; lane i receives
 // E[i/4][i%4], E[4 + i/4][i%4], E[8 + i/4][i%4], E[12 + i/4][i%4].  With lane 4r+q pointing at columns 4q..4q+3 of row r
 // of a 4 x 16 block, lane i receives column i of the four rows.
@@ -195,8 +183,13 @@ G4B_DEV u2 lds_read8_tr16(uint32_t lds_addr, int imm) {
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(imm));
     return v;
 }
+// Wait until at most N LDS operations are outstanding; the values are tied so their consumers stay behind the wait.
 template <int N>
-G4B_DEV void lds_wait2(u2& a, u2& b) {
+G4B_DEV void lds_wait4(u2& a, u2& b, u2& c, u2& d) {
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+G4B_DEV void lds_wait_pair(u4& a, u4& b) {
     asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
 

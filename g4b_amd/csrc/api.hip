@@ -28,6 +28,23 @@ bool dtype_ok(int dt) { return dt == G4B_DT_F16 || dt == G4B_DT_BF16 || dt == G4
 
 uint64_t decode_slots(int B, int G, int nw) { return (uint64_t)nw + (uint64_t)B * G; }
 
+// Prefill-shaped launches: how many (active slot, key split) pairs the partial buffers hold.  A launch whose in-phase
+// slots bring fewer workgroups than the chip has CUs splits the keys of every item; 0 = the shape never splits.
+constexpr int kPrefillFillWorkgroups = 256;
+constexpr int kPrefillMaxSplitSlots = 64;
+int prefill_split_slots(int H, int G, int Tq) {
+    const int R = H / G;
+    if (R < 1 || 128 % R) return 0;
+    const int tokb = 128 / R;
+    const int64_t per_slot = (int64_t)((Tq + tokb - 1) / tokb) * G;  // workgroups one slot brings
+    const int64_t slots = kPrefillFillWorkgroups / per_slot;
+    if (slots < 2) return 0;
+    return (int)(slots < kPrefillMaxSplitSlots ? slots : kPrefillMaxSplitSlots);
+}
+uint64_t prefill_workspace_bytes(int H, int G, int Tq, int D) {
+    return (uint64_t)prefill_split_slots(H, G, Tq) * (uint64_t)H * (uint64_t)Tq * (uint64_t)(D + 2) * sizeof(float);
+}
+
 }  // namespace
 
 extern "C" {
@@ -39,7 +56,7 @@ int32_t g4b_attn_default_workers(void) { return kDefaultWorkers; }
 uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers) {
     if (B < 1 || H < 1 || G < 1 || Tq < 1 || D < 1 || H % G) return 0;
     const int64_t rows = (int64_t)(H / G) * Tq;
-    if (rows > kMaxDecodeRows) return 0;
+    if (rows > kMaxDecodeRows) return prefill_workspace_bytes(H, G, Tq, D);
     const int nw = num_workers > 0 ? num_workers : kDefaultWorkers;
     return decode_slots(B, G, nw) * (uint64_t)rows * (uint64_t)(D + 2) * sizeof(float);
 }
@@ -131,6 +148,17 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
         if (128 % p.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide 128 for prefill-shaped launches", p.R);
+        p.split_slots = 0;
+        const uint64_t need = prefill_workspace_bytes(a->H, a->G, a->Tq, a->D);
+        if (a->workspace && need) {
+            if (a->workspace_bytes < need)
+                return fail(G4B_ERR_WORKSPACE, "workspace holds %llu bytes, %llu needed to split this prefill shape",
+                            (unsigned long long)a->workspace_bytes, (unsigned long long)need);
+            if (!aligned16(a->workspace)) return fail(G4B_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+            p.split_slots = prefill_split_slots(a->H, a->G, a->Tq);
+            p.part_o = static_cast<float*>(a->workspace);
+            p.part_ml = p.part_o + (uint64_t)p.split_slots * a->H * a->Tq * a->D;
+        }
         e = g4b::launch_attn_prefill(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     }
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));

@@ -84,7 +84,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     // by their linear id and every XCD has an L2 of its own, so the ids are mapped such that an XCD walks the K/V of
     // as few heads as possible, its workgroups start at the same key and advance together (one fetch from memory
     // serves the XCD), the heaviest (latest) query tiles start first, and the XCDs get equal shares.
-    const PfMap map = pf_map(p.G * p.B, (Tq + TOKB - 1) / TOKB);
+    // The work list is built from the slots that are in phase, so a launch with few of them (one prefill chunk in a
+    // batch of decoding slots) can split every item's keys over several workgroups and still fill the chip.
+    __shared__ int sh_scan[8];
+    int n_active;
+    nth_active_slot(p, -1, n_active, sh_scan);
+    if (n_active == 0) return;
+    const int nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
+    const PfMap map = pf_map(n_active * p.G * nsplit, (Tq + TOKB - 1) / TOKB);
+    if ((int)blockIdx.x >= map.grid) return;
     int head, rank;
     {
         const int f = blockIdx.x, x = f & 7, j = f >> 3;
@@ -101,10 +109,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     }
     if (rank >= map.nq) return;
     const int qtile = map.nq - 1 - rank;
-    const int g = head % p.G, b = head / p.G;
+    const int split = head % nsplit, g = (head / nsplit) % p.G, a_idx = head / (nsplit * p.G);
+    const int b = nth_active_slot(p, a_idx, n_active, sh_scan);  // workgroup-uniform
 
     const SlotInfo si = slot_info(p, b);
-    if (!si.active) return;
 
     const int tok0 = qtile * TOKB;
     const int tok_last = min(tok0 + TOKB, Tq) - 1;
@@ -250,7 +258,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             else lds_wait4<0>(f0.lo, f0.hi, f1.lo, f1.hi);
         };
 
-        const int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
+        // this workgroup's share of the item's key tiles
+        int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
+        if (nsplit > 1) {
+            const int n = kt1 - kt0 + 1;
+            kt1 = kt0 + (split + 1) * n / nsplit - 1;
+            kt0 = kt0 + split * n / nsplit;
+        }
+        if (kt1 >= kt0) {
 
         // ---- prologue: K(kt0), K(kt0+1), V(kt0) staged; S(kt0) computed --------------------------------
         stage_whole_tile(kt0, false, 0);
@@ -426,26 +441,87 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             s_cur[0] = s_nxt[0];
             s_cur[1] = s_nxt[1];
         }
+        }
     }
 
     // ---- epilogue: lane (row n32, half h2) holds d = 32*dt + 8*(i/4) + 4*h2 + i%4 -----------------
     const float l_tot = half_swap_sum(l_run);
-    if (row_ok) {
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (!row_ok) return;
+    if (nsplit > 1) {
+        // un-normalised partial result of this key split: [pair][H][Tq][D] fp32 and (reference, sum) per row
+        const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hh)) * Tq + ti;
+        float* po = p.part_o + prow * D;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                f4 v = {acc[dt][4 * q4] * inv, acc[dt][4 * q4 + 1] * inv, acc[dt][4 * q4 + 2] * inv, acc[dt][4 * q4 + 3] * inv};
-                store4(p.o, ooff + dt * 32 + 8 * q4 + 4 * h2, p.o_dt, v);
+                f4 v = {acc[dt][4 * q4], acc[dt][4 * q4 + 1], acc[dt][4 * q4 + 2], acc[dt][4 * q4 + 3]};
+                *reinterpret_cast<f4*>(po + dt * 32 + 8 * q4 + 4 * h2) = v;
             }
+        if (h2 == 0) {
+            p.part_ml[prow * 2] = (m_run == -INFINITY) ? 0.f : m_run;
+            p.part_ml[prow * 2 + 1] = l_tot;
+        }
+        return;
+    }
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            f4 v = {acc[dt][4 * q4] * inv, acc[dt][4 * q4 + 1] * inv, acc[dt][4 * q4 + 2] * inv, acc[dt][4 * q4 + 3] * inv};
+            store4(p.o, ooff + dt * 32 + 8 * q4 + 4 * h2, p.o_dt, v);
+        }
+}
+
+// Merge the key splits of a prefill-shaped launch: one workgroup per (active slot, query head, 32 tokens), four
+// rows at a time, a lane per four output columns.
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
+    __shared__ int sh_scan[8];
+    const int tblocks = (p.Tq + 31) / 32;
+    const int a_idx = blockIdx.x / (p.H * tblocks), h = (blockIdx.x / tblocks) % p.H, tb = blockIdx.x % tblocks;
+    int n_active;
+    const int b = nth_active_slot(p, a_idx, n_active, sh_scan);
+    const int nsplit = prefill_splits(p.split_slots, n_active);
+    if (b < 0 || nsplit == 1) return;
+    constexpr int LPR = D / 4;         // lanes per row
+    constexpr int RPP = 256 / LPR;     // rows per pass
+    const int r_in = threadIdx.x / LPR, d0 = (threadIdx.x % LPR) * 4;
+    for (int t = tb * 32 + r_in; t < min(tb * 32 + 32, p.Tq); t += RPP) {
+        float mref = -INFINITY;
+        for (int s = 0; s < nsplit; ++s) {
+            const float* ml = p.part_ml + ((((int64_t)(a_idx * nsplit + s) * p.H + h) * p.Tq + t) * 2);
+            if (ml[1] > 0.f) mref = fmaxf(mref, ml[0]);
+        }
+        f4 acc = {0.f, 0.f, 0.f, 0.f};
+        float l = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const int64_t prow = ((int64_t)(a_idx * nsplit + s) * p.H + h) * p.Tq + t;
+            const float ms = p.part_ml[prow * 2], ls = p.part_ml[prow * 2 + 1];
+            if (ls > 0.f) {
+                const float w = fast_exp2(ms - mref);
+                const f4 v = *reinterpret_cast<const f4*>(p.part_o + prow * D + d0);
+                acc += v * w;
+                l += ls * w;
+            }
+        }
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)h * p.o_s[1] + (int64_t)t * p.o_s[2] + d0;
+        store4(p.o, ooff, p.o_dt, acc * inv);
     }
 }
 
 template <int D, class T>
 static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     const int TOKB = PF_BM / p.R;
-    dim3 grid(pf_map(p.G * p.B, (p.Tq + TOKB - 1) / TOKB).grid);
+    // The grid is sized for the worst case over the number of slots that turn out to be in phase; the kernel reads
+    // that number on the device and surplus workgroups leave at once.
+    const int nq = (p.Tq + TOKB - 1) / TOKB;
+    const int slots = p.part_o ? p.split_slots : 1;
+    int blocks = 0;
+    for (int n = 1; n <= p.B; ++n) blocks = max(blocks, pf_map(n * p.G * prefill_splits(slots, n), nq).grid);
+    dim3 grid(blocks);
     const int smem = 4 * PfSmem<D>::TILE;
     static bool attr_set = false;
     if (!attr_set) {
@@ -454,7 +530,11 @@ static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((attn_prefill_kernel<D, T>), grid, dim3(256), smem, stream, p);
+    if (p.kernel_mask & 1) hipLaunchKernelGGL((attn_prefill_kernel<D, T>), grid, dim3(256), smem, stream, p);
+    if (slots > 1 && (p.kernel_mask & 2)) {
+        const int items = min(p.B, slots / 2);  // more active slots than this are never split
+        hipLaunchKernelGGL((attn_prefill_combine<D>), dim3(items * p.H * ((p.Tq + 31) / 32)), dim3(256), 0, stream, p);
+    }
     return hipGetLastError();
 }
 

@@ -224,6 +224,7 @@ struct AttnParams {
     int32_t B, H, G, R, Tq, KV_CTX;
     int32_t W, phase, stage, qwin;
     int32_t NW;  // number of decode workers (waves) the key tiles are dealt to
+    int32_t split_slots;  // prefill: (active slot, key split) pairs the partial buffers hold; <= 1 = never split
     int32_t kernel_mask;  // bit 0: main kernel, bit 1: merge kernel
     float c;     // softmax scale * log2(e)
 };
@@ -251,6 +252,37 @@ G4B_DEV SlotInfo slot_info(const AttnParams& p, int b) {
     if (p.qwin > 0) klo = min(max(0, s.qb - p.qwin + 1), s.window);
     s.klo = klo;
     return s;
+}
+
+// Number of slots whose phase matches the launch (n_active) and the index of the a-th of them (-1 when a is out of
+// range).  Every thread of a 256-thread workgroup must call it; sh is workgroup-shared scratch of at least 5 ints.
+// Call it with a < 0 to count only.
+G4B_DEV int nth_active_slot(const AttnParams& p, int a, int& n_active, int* sh) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int base = 0;
+    for (int c0 = 0; c0 < p.B; c0 += 256) {
+        const int b = c0 + tid;
+        const bool act = b < p.B && p.phase_arr[(int64_t)b * p.ph_s] == (uint8_t)p.phase;
+        const unsigned long long m = __ballot(act);
+        if (lane == 0) sh[wave] = __popcll(m);
+        __syncthreads();
+        int before = base;
+        for (int w = 0; w < wave; ++w) before += sh[w];
+        const int total = sh[0] + sh[1] + sh[2] + sh[3];
+        const int rank = before + __popcll(m & ((1ull << lane) - 1ull));
+        if (act && rank == a) sh[4] = b;
+        base += total;
+        __syncthreads();
+    }
+    n_active = base;
+    return (a >= 0 && a < base) ? sh[4] : -1;
+}
+
+// Key splits per active slot of a prefill-shaped launch: the partial buffers hold split_slots (slot, split) pairs.
+__host__ __device__ inline int prefill_splits(int split_slots, int n_active) {
+    if (n_active < 1 || split_slots < 2 * n_active) return 1;
+    const int s = split_slots / n_active;
+    return s < 16 ? s : 16;
 }
 
 // Visible logical key range [lo, hi) of query i of a slot.

@@ -31,7 +31,8 @@ _private_workspaces: dict = {}
 
 
 def workspace_bytes(B: int, H: int, G: int, Tq: int, D: int, num_workers: int = 0) -> int:
-    """Bytes of scratch a decode-shaped launch needs to split keys over ``num_workers`` waves."""
+    """Bytes of scratch that let a launch of this shape split keys: over ``num_workers`` waves when it is
+    decode-shaped, over workgroups when it is a prefill shape that would not fill the chip (0 otherwise)."""
     return int(_native.load().g4b_attn_workspace_bytes(B, H, G, Tq, D, num_workers))
 
 
@@ -103,7 +104,7 @@ def flash_attention(
     * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
       ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
       ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
-      used for split partials instead of the private one); ``num_workers``; ``kernel_mask`` (profiling:
+      used for split partials instead of the private one; ``False`` = use none and never split); ``num_workers``; ``kernel_mask`` (profiling:
       bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
 
     Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
@@ -175,9 +176,18 @@ def flash_attention(
     a.kernel_mask = int(kernel_mask)
     a.scale = float(scale)
 
-    ws = workspace
-    if ws is None and max_kv_splits > 1 and (H // G) * Tq <= MAX_DECODE_ROWS:
-        ws = _private_workspace(q, workspace_bytes(B, H, G, Tq, D, num_workers))
+    ws = None if workspace is False else workspace
+    if workspace is False:
+        pass  # no scratch at all: nothing is split
+    elif ws is None and (H // G) * Tq <= MAX_DECODE_ROWS:
+        if max_kv_splits > 1:
+            ws = _private_workspace(q, workspace_bytes(B, H, G, Tq, D, num_workers))
+    elif ws is None:
+        # prefill-shaped: shapes whose in-phase slots may bring fewer workgroups than the chip has CUs
+        # (chunked prefill, short prompts) split every item's keys and merge; other shapes need none
+        need = workspace_bytes(B, H, G, Tq, D, 0)
+        if need:
+            ws = _private_workspace(q, need)
     if ws is not None:
         a.workspace = ws.data_ptr()
         a.workspace_bytes = int(ws.numel()) * int(ws.element_size()) if hasattr(ws, "numel") else int(ws.nbytes)

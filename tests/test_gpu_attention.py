@@ -113,6 +113,64 @@ def test_prefill_matches_oracle(fa, case, scale):
     assert_close(o.float().cpu().numpy(), ref, what=name)
 
 
+@pytest.mark.parametrize("case", PREFILL_CASES[:3] + PREFILL_CASES[4:5], ids=[c[0] for c in PREFILL_CASES[:3] + PREFILL_CASES[4:5]])
+def test_prefill_key_split_agrees_with_one_workgroup_per_tile(fa, case):
+    """Shapes that bring few workgroups split every item's keys over several and merge the partials; with
+    ``workspace=False`` nothing is split.  Both must match the oracle and each other."""
+    name, B, H, G, Tq, kv_ctx, D, W, stage = case
+    assert fa.workspace_bytes(B, H, G, Tq, D) > 0, "these shapes are meant to take the split path"
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=14)
+    tds = [W if b % 2 == 0 else W + 17 for b in range(B)]
+    ref = oracle(q, k, v, tds, [1] * B, W, 1, stage=stage, scale=1 / 16)
+    fa.flash_attention(q, k, v, o, i32(tds), u8([1] * B), W, 1, stage=stage, scale=1 / 16)
+    o1 = torch.full_like(o, 777.0)
+    fa.flash_attention(q, k, v, o1, i32(tds), u8([1] * B), W, 1, stage=stage, scale=1 / 16, workspace=False)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what=f"{name} split")
+    assert_close(o1.float().cpu().numpy(), ref, what=f"{name} unsplit")
+    diff = (o1.float() - o.float()).abs()
+    assert bool((diff <= 5e-4 + 2e-3 * o.float().abs()).all()), diff.max().item()
+
+
+@pytest.mark.parametrize("n_prefill", [1, 2, 5, 9])
+def test_prefill_chunk_inside_a_mixed_batch(fa, n_prefill):
+    """The engine's mixed step: a few slots prefill a chunk while the others decode or are unallocated.  The number of
+    key splits follows the number of in-phase slots, which only the device knows."""
+    B, H, G, Tq, D, W = 9, 8, 2, 96, 256, 3000
+    kv_ctx = W + Tq - 1
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=15)
+    order = [4, 0, 8, 2, 6, 1, 3, 5, 7]
+    phase = [2 if b % 2 else 0 for b in range(B)]
+    for b in order[:n_prefill]:
+        phase[b] = 1
+    tds = [Tq + 37 * b * b * 3 for b in range(B)]  # from a bare chunk to a wrapped ring
+    tds[order[0]] = 5000 + Tq
+    ref = oracle(q, k, v, tds, phase, W, 1, scale=1 / 16)
+    o.fill_(123.0)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, scale=1 / 16)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(got[b], ref[b], what=f"slot {b} of {n_prefill} prefilling")
+        else:
+            assert (got[b] == 123.0).all(), f"off-phase slot {b} was written"
+
+
+def test_prefill_workspace_too_small_is_refused(fa):
+    B, H, G, Tq, D, W = 1, 8, 2, 128, 256, 1024
+    q, k, v, o = make_case(B, H, G, Tq, D, W, seed=16)
+    need = fa.workspace_bytes(B, H, G, Tq, D)
+    assert need > 0
+    small = torch.empty(need - 16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(ValueError, match="workspace"):
+        fa.flash_attention(q, k, v, o, i32([W]), u8([1]), W, 1, workspace=small)
+    exact = torch.empty(need, dtype=torch.uint8, device="cuda")
+    fa.flash_attention(q, k, v, o, i32([W]), u8([1]), W, 1, scale=1 / 16, workspace=exact)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), oracle(q, k, v, [W], [1], W, 1, scale=1 / 16), what="caller workspace")
+
+
 def test_one_shot_causal_prefill_2048(fa):
     """BASELINE config 2: batch 1, seq 2048, 8 q heads / 2 kv heads, head dim 256, scale 1/16."""
     B, H, G, Tq, D = 1, 8, 2, 2048, 256

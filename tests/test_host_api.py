@@ -78,7 +78,12 @@ def test_workspace_size_formula(native):
     # (workers + B*G) partial slots of rows x (D + 2) floats
     assert lib.g4b_attn_workspace_bytes(64, 8, 2, 1, 256, 0) == (nw + 128) * 4 * 258 * 4
     assert lib.g4b_attn_workspace_bytes(3, 8, 2, 2, 128, 10) == (10 + 6) * 8 * 130 * 4
-    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 512, 256, 0) == 0  # prefill-shaped: no workspace
+    # prefill-shaped: (slot, key split) pairs x H x Tq rows x (D + 2) floats when one slot brings fewer than 256
+    # workgroups (16 query tiles x 2 kv heads here -> 8 pairs), nothing when the shape fills the chip by itself
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 512, 256, 0) == 8 * 8 * 512 * 258 * 4
+    assert lib.g4b_attn_workspace_bytes(33, 8, 2, 512, 256, 0) == 8 * 8 * 512 * 258 * 4  # independent of B
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 2048, 256, 0) == 2 * 8 * 2048 * 258 * 4
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 8192, 256, 0) == 0
 
 
 def _decode_args():

@@ -279,51 +279,38 @@ __global__ __launch_bounds__(64, 1) void attn_decode_worker(const AttnParams p) 
     }
 }
 
-// Merge the partials of each (slot, kv head) pair; one workgroup per pair, 256 threads.
+// Merge the partials of each (slot, kv head) pair: one workgroup of 256 threads per (pair, query row).  The workers
+// that own tiles of the pair are spread over the four waves and their loads are independent, so the merge costs a few
+// memory round trips however many workers a long slot was dealt to.
 template <int D>
 __global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
-    __shared__ int red[256];
-    const int tid = threadIdx.x;
-    const int pair = blockIdx.x;
+    __shared__ float sm_max[4];
+    __shared__ float sm_l[4];
+    __shared__ f4 sm_acc[4][D / 4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pair = blockIdx.x, row = blockIdx.y;
     const int b = pair / p.G, g = pair % p.G;
     const int B = p.B, G = p.G;
     const int NR = p.R * p.Tq;
 
-    // flat start of this pair and total tile count (same arithmetic as the workers)
+    // flat start of this pair and total tile count (same arithmetic as the workers), computed by every wave
     int before = 0, total = 0;
-    for (int x = tid; x < B; x += 256) {
-        int c = G * slot_tiles(p, x);
+    for (int b0 = 0; b0 < B; b0 += 64) {
+        const int x = b0 + lane;
+        const int c = (x < B) ? G * slot_tiles(p, x) : 0;
         total += c;
-        if (x < b) before += c;
+        before += (x < b) ? c : 0;
     }
-    red[tid] = before;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (tid < o) red[tid] += red[tid + o];
-        __syncthreads();
-    }
-    before = red[0];
-    __syncthreads();
-    red[tid] = total;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (tid < o) red[tid] += red[tid + o];
-        __syncthreads();
-    }
-    total = red[0];
+    total = wave_sum_i(total);
+    before = wave_sum_i(before);
 
     const SlotInfo si = slot_info(p, b);
     if (!si.active) return;
     const int tl = slot_tiles(p, b);
-    const int nvec = NR * (D / 4);
+    const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] + (int64_t)(row % p.Tq) * p.o_s[2];
     if (tl == 0) {
         // in-phase slot without any visible key: defined as zeros
-        for (int x = tid; x < nvec; x += 256) {
-            const int row = x / (D / 4), d0 = (x % (D / 4)) * 4;
-            const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] +
-                                 (int64_t)(row % p.Tq) * p.o_s[2] + d0;
-            store4(p.o, ooff, p.o_dt, f4{0.f, 0.f, 0.f, 0.f});
-        }
+        if (tid < D / 4) store4(p.o, ooff + tid * 4, p.o_dt, f4{0.f, 0.f, 0.f, 0.f});
         return;
     }
     if (p.NW == 0) return;  // one wave owned the whole pair
@@ -334,26 +321,53 @@ __global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
     const int w1 = (int)(((fs + tl) * nw - 1) / total);
     if (w0 == w1) return;  // a single worker owned the pair and wrote the output itself
 
-    for (int x = tid; x < nvec; x += 256) {
-        const int row = x / (D / 4), d0 = (x % (D / 4)) * 4;
-        float m = -INFINITY, l = 0.f;
-        f4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int w = w0; w <= w1; ++w) {
-            const int64_t slot = (int64_t)w + pair;
-            const float* pm = p.part_ml + (slot * NR + row) * 2;
-            const float mw = pm[0], lw = pm[1];
-            if (mw == -INFINITY) continue;
-            const f4 ow = *reinterpret_cast<const f4*>(p.part_o + (slot * NR + row) * D + d0);
-            const float mn = fmaxf(m, mw);
-            const float a = fast_exp2(m - mn), bw = fast_exp2(mw - mn);
-            acc = acc * a + ow * bw;
-            l = l * a + lw * bw;
-            m = mn;
+    // partial of worker w for this pair and row: slot w + pair
+    auto ml_of = [&](int w) { return p.part_ml + (((int64_t)w + pair) * NR + row) * 2; };
+    // pass 1: the row's reference = largest reference any worker used (-inf marks a worker without keys for the row)
+    float mref = -INFINITY;
+    for (int w = w0 + tid; w <= w1; w += 256) mref = fmaxf(mref, ml_of(w)[0]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mref = fmaxf(mref, __shfl_xor(mref, o));
+    if (lane == 0) sm_max[wave] = mref;
+    __syncthreads();
+    mref = fmaxf(fmaxf(sm_max[0], sm_max[1]), fmaxf(sm_max[2], sm_max[3]));
+    const float msafe = (mref == -INFINITY) ? 0.f : mref;
+
+    // pass 2: wave k takes workers w0 + k, w0 + k + 4, ...; a lane owns four output columns
+    constexpr int LPR = D / 4;  // lanes that hold a row
+    constexpr int UN = 8;
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.f;
+    for (int wb = w0 + wave; wb <= w1; wb += 4 * UN) {
+        float wgt[UN], lw[UN];
+        f4 ov[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int w = min(wb + 4 * u, w1);  // clamped loads, masked below
+            const float* ml = ml_of(w);
+            wgt[u] = ml[0];
+            lw[u] = ml[1];
+            ov[u] = (lane < LPR) ? *reinterpret_cast<const f4*>(p.part_o + (((int64_t)w + pair) * NR + row) * D + lane * 4)
+                                 : f4{0.f, 0.f, 0.f, 0.f};
         }
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] +
-                             (int64_t)(row % p.Tq) * p.o_s[2] + d0;
-        store4(p.o, ooff, p.o_dt, acc * inv);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const bool live = (wb + 4 * u <= w1) && (wgt[u] != -INFINITY);
+            const float e = live ? fast_exp2(wgt[u] - msafe) : 0.f;
+            if (live) {
+                acc += ov[u] * e;
+                l += lw[u] * e;
+            }
+        }
+    }
+    if (lane < LPR) sm_acc[wave][lane] = acc;
+    if (lane == 0) sm_l[wave] = l;
+    __syncthreads();
+    if (tid < LPR) {
+        const f4 r = sm_acc[0][tid] + sm_acc[1][tid] + sm_acc[2][tid] + sm_acc[3][tid];
+        const float lt = sm_l[0] + sm_l[1] + sm_l[2] + sm_l[3];
+        const float inv = lt > 0.f ? 1.f / lt : 0.f;
+        store4(p.o, ooff + tid * 4, p.o_dt, r * inv);
     }
 }
 
@@ -364,7 +378,7 @@ static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (p.kernel_mask & 2) hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G), dim3(256), 0, stream, p);
+    if (p.kernel_mask & 2) hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G, p.R * p.Tq), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -140,14 +140,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     float m_run = -INFINITY, l_run = 0.f;  // exponent reference in log2 units (scaled), running sum (this lane's keys)
 
     if (hi_wg > lo_wg) {
-        // Q as B operand: lane (row n32, half h2), step c: d = 16c + 8*h2 .. +8
-        u4 qf[KSTEPS];
-#pragma unroll
-        for (int c = 0; c < KSTEPS; ++c) {
-            u4 z = {0, 0, 0, 0};
-            qf[c] = row_ok ? load8_as<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt) : z;
-        }
-
         const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
         const char* vbase = static_cast<const char*>(p.v) + ((int64_t)b * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
         auto key_off = [&](int j) -> uint32_t {  // byte offset of logical key j (clamped to the window) in the ring
@@ -271,6 +263,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
         stage_whole_tile(kt0, false, 0);
         stage_whole_tile(kt0 + 1, false, 1);
         stage_whole_tile(kt0, true, 0);
+        // Q as B operand: lane (row n32, half h2), step c: d = 16c + 8*h2 .. +8 (loaded behind the staging loads)
+        u4 qf[KSTEPS];
+#pragma unroll
+        for (int c = 0; c < KSTEPS; ++c) {
+            u4 z = {0, 0, 0, 0};
+            qf[c] = row_ok ? load8_as<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt) : z;
+        }
         vm_wait_all();
         __syncthreads();
         f16v s_cur[2];
@@ -474,42 +473,59 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
         }
 }
 
-// Merge the key splits of a prefill-shaped launch: one workgroup per (active slot, query head, 32 tokens), four
-// rows at a time, a lane per four output columns.
+// Merge the key splits of a prefill-shaped launch: a lane per four output columns of a row, PFC_ROWS rows per
+// workgroup, every load of a row independent of the others.
+constexpr int PFC_ROWS = 8;
+template <int D, int NS>
+G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, int tb, int nsplit) {
+    constexpr int LPR = D / 4;      // lanes per row
+    constexpr int RPP = 256 / LPR;  // rows per pass
+    const int r_in = threadIdx.x / LPR, d0 = (threadIdx.x % LPR) * 4;
+#pragma unroll
+    for (int pass = 0; pass < PFC_ROWS / RPP; ++pass) {
+        const int t = tb * PFC_ROWS + pass * RPP + r_in;
+        if (t >= p.Tq) continue;
+        float ms[NS], ls[NS];
+        f4 ov[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int64_t prow = ((int64_t)(a_idx * nsplit + min(s, nsplit - 1)) * p.H + h) * p.Tq + t;  // clamped, masked below
+            ms[s] = p.part_ml[prow * 2];
+            ls[s] = (s < nsplit) ? p.part_ml[prow * 2 + 1] : 0.f;
+            ov[s] = *reinterpret_cast<const f4*>(p.part_o + prow * D + d0);
+        }
+        float mref = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (ls[s] > 0.f) mref = fmaxf(mref, ms[s]);
+        f4 acc = {0.f, 0.f, 0.f, 0.f};
+        float l = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (ls[s] > 0.f) {
+                const float w = fast_exp2(ms[s] - mref);
+                acc += ov[s] * w;
+                l += ls[s] * w;
+            }
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)h * p.o_s[1] + (int64_t)t * p.o_s[2] + d0;
+        store4(p.o, ooff, p.o_dt, acc * inv);
+    }
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
     __shared__ int sh_scan[8];
-    const int tblocks = (p.Tq + 31) / 32;
+    const int tblocks = (p.Tq + PFC_ROWS - 1) / PFC_ROWS;
     const int a_idx = blockIdx.x / (p.H * tblocks), h = (blockIdx.x / tblocks) % p.H, tb = blockIdx.x % tblocks;
     int n_active;
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);
     const int nsplit = prefill_splits(p.split_slots, n_active);
     if (b < 0 || nsplit == 1) return;
-    constexpr int LPR = D / 4;         // lanes per row
-    constexpr int RPP = 256 / LPR;     // rows per pass
-    const int r_in = threadIdx.x / LPR, d0 = (threadIdx.x % LPR) * 4;
-    for (int t = tb * 32 + r_in; t < min(tb * 32 + 32, p.Tq); t += RPP) {
-        float mref = -INFINITY;
-        for (int s = 0; s < nsplit; ++s) {
-            const float* ml = p.part_ml + ((((int64_t)(a_idx * nsplit + s) * p.H + h) * p.Tq + t) * 2);
-            if (ml[1] > 0.f) mref = fmaxf(mref, ml[0]);
-        }
-        f4 acc = {0.f, 0.f, 0.f, 0.f};
-        float l = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const int64_t prow = ((int64_t)(a_idx * nsplit + s) * p.H + h) * p.Tq + t;
-            const float ms = p.part_ml[prow * 2], ls = p.part_ml[prow * 2 + 1];
-            if (ls > 0.f) {
-                const float w = fast_exp2(ms - mref);
-                const f4 v = *reinterpret_cast<const f4*>(p.part_o + prow * D + d0);
-                acc += v * w;
-                l += ls * w;
-            }
-        }
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)h * p.o_s[1] + (int64_t)t * p.o_s[2] + d0;
-        store4(p.o, ooff, p.o_dt, acc * inv);
-    }
+    if (nsplit <= 2) prefill_combine_rows<D, 2>(p, a_idx, b, h, tb, nsplit);
+    else if (nsplit <= 4) prefill_combine_rows<D, 4>(p, a_idx, b, h, tb, nsplit);
+    else if (nsplit <= 8) prefill_combine_rows<D, 8>(p, a_idx, b, h, tb, nsplit);
+    else prefill_combine_rows<D, 16>(p, a_idx, b, h, tb, nsplit);
 }
 
 template <int D, class T>
@@ -533,7 +549,7 @@ static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     if (p.kernel_mask & 1) hipLaunchKernelGGL((attn_prefill_kernel<D, T>), grid, dim3(256), smem, stream, p);
     if (slots > 1 && (p.kernel_mask & 2)) {
         const int items = min(p.B, slots / 2);  // more active slots than this are never split
-        hipLaunchKernelGGL((attn_prefill_combine<D>), dim3(items * p.H * ((p.Tq + 31) / 32)), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((attn_prefill_combine<D>), dim3(items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS)), dim3(256), 0, stream, p);
     }
     return hipGetLastError();
 }

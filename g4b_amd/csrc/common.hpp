@@ -259,6 +259,14 @@ G4B_DEV SlotInfo slot_info(const AttnParams& p, int b) {
 // Call it with a < 0 to count only.
 G4B_DEV int nth_active_slot(const AttnParams& p, int a, int& n_active, int* sh) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (p.B <= 64) {  // one ballot per wave answers both questions, no exchange between waves
+        const bool act = lane < p.B && p.phase_arr[(int64_t)lane * p.ph_s] == (uint8_t)p.phase;
+        const unsigned long long m = __ballot(act);
+        n_active = __popcll(m);
+        if (a < 0 || a >= n_active) return -1;
+        const unsigned long long hit = __ballot(act && __popcll(m & ((1ull << lane) - 1ull)) == a);
+        return __ffsll((long long)hit) - 1;
+    }
     int base = 0;
     for (int c0 = 0; c0 < p.B; c0 += 256) {
         const int b = c0 + tid;

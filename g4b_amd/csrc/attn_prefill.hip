@@ -130,7 +130,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     if (row_ok) row_range(p, si, ti, lo_r, hi_r);
 
     const int64_t qoff = (int64_t)b * p.q_s[0] + (int64_t)(g * R + hh) * p.q_s[1] + (int64_t)ti * p.q_s[2];
-    const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hh) * p.o_s[1] + (int64_t)ti * p.o_s[2];
 
     f16v acc[DT];
 #pragma unroll
@@ -443,34 +442,49 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
         }
     }
 
-    // ---- epilogue: lane (row n32, half h2) holds d = 32*dt + 8*(i/4) + 4*h2 + i%4 -----------------
+    // ---- epilogue ---------------------------------------------------------------------------------------
+    // Lane (row n32, half h2) holds columns d = 32*dt + 8*(i/4) + 4*h2 + i%4 of its row.  The wave turns its 32 x D
+    // block around in LDS (its own 32 * D * 4 bytes of the staging area, free after the loop's last barrier; 16-byte
+    // pieces XOR-swizzled with the row so that neither side conflicts) and stores whole rows: one instruction covers
+    // 64 / (D/4) complete rows instead of touching 32 rows at 8 or 16 bytes each.
     const float l_tot = half_swap_sum(l_run);
-    if (!row_ok) return;
-    if (nsplit > 1) {
-        // un-normalised partial result of this key split: [pair][H][Tq][D] fp32 and (reference, sum) per row
-        const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hh)) * Tq + ti;
-        float* po = p.part_o + prow * D;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                f4 v = {acc[dt][4 * q4], acc[dt][4 * q4 + 1], acc[dt][4 * q4 + 2], acc[dt][4 * q4 + 3]};
-                *reinterpret_cast<f4*>(po + dt * 32 + 8 * q4 + 4 * h2) = v;
-            }
-        if (h2 == 0) {
-            p.part_ml[prow * 2] = (m_run == -INFINITY) ? 0.f : m_run;
-            p.part_ml[prow * 2 + 1] = l_tot;
-        }
-        return;
-    }
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const bool partial = nsplit > 1;
+    const float inv = partial ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);
+    char* wbase = smem + wave * (32 * D * 4);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
             f4 v = {acc[dt][4 * q4] * inv, acc[dt][4 * q4 + 1] * inv, acc[dt][4 * q4 + 2] * inv, acc[dt][4 * q4 + 3] * inv};
-            store4(p.o, ooff + dt * 32 + 8 * q4 + 4 * h2, p.o_dt, v);
+            const int pc = 8 * dt + 2 * q4 + h2;
+            *reinterpret_cast<f4*>(wbase + n32 * (D * 4) + ((pc ^ (n32 & 15)) * 16)) = v;
         }
+    if (partial && h2 == 0 && row_ok) {
+        // (reference, sum) of this key split's rows
+        const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hh)) * Tq + ti;
+        p.part_ml[prow * 2] = (m_run == -INFINITY) ? 0.f : m_run;
+        p.part_ml[prow * 2 + 1] = l_tot;
+    }
+    constexpr int LPR = D / 4;       // lanes that cover a row, 16 bytes of fp32 each
+    constexpr int RPI = 64 / LPR;    // rows per store instruction
+    const int tokb_shift = __ffs(TOKB) - 1;  // TOKB = 128 / R is a power of two
+#pragma unroll 4
+    for (int i = 0; i < 32 / RPI; ++i) {
+        const int row = i * RPI + lane / LPR, pc = lane % LPR;
+        const int rr = wave * 32 + row;
+        const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
+        const f4 v = *reinterpret_cast<const f4*>(wbase + row * (D * 4) + ((pc ^ (row & 15)) * 16));
+        if (tr < Tq) {
+            if (partial) {
+                // un-normalised partial result of this key split: [pair][H][Tq][D] fp32
+                const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
+                *reinterpret_cast<f4*>(p.part_o + prow * D + pc * 4) = v;
+            } else {
+                const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
+                store4(p.o, off + pc * 4, p.o_dt, v);
+            }
+        }
+    }
 }
 
 // Merge the key splits of a prefill-shaped launch: a lane per four output columns of a row, PFC_ROWS rows per

@@ -61,13 +61,17 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *                 reference's one-shot prefill (scripts/reference_impl.py:440-441).
  *   window_sizes  optional [B] int32 per-slot override of ctx_window_size (extension; NULL = none).
  *   workspace     device scratch for split-KV partials, >= g4b_attn_workspace_bytes(...) bytes, or
- *                 NULL: then a decode-shaped launch (R*Tq <= 16) uses one wave per (slot, kv head).
- *                 Contents are unspecified after the call (like partial_o/l/m, fa2.py:643-645).
+ *                 NULL: then a decode-shaped launch (R*Tq <= 16) uses one wave per (slot, kv head)
+ *                 and a prefill-shaped launch one workgroup per (slot, kv head, query tile) however
+ *                 few slots are in phase.  Contents are unspecified after the call (like
+ *                 partial_o/l/m, fa2.py:643-645).
  *   num_workers   0 = library default; otherwise the number of waves the decode key tiles are
- *                 dealt to (must not exceed the value the workspace was sized for).
+ *                 dealt to (must not exceed the value the workspace was sized for).  Ignored by
+ *                 prefill-shaped launches, which choose their key split from the number of in-phase
+ *                 slots on the device.
  *   kernel_mask   profiling aid.  0 = run every kernel of the launch.  Otherwise bit 0 selects the
- *                 main attention kernel and bit 1 the split-merge kernel of a decode-shaped launch,
- *                 so that each can be timed on its own; results are only complete with both.
+ *                 main attention kernel and bit 1 the split-merge kernel, so that each can be timed
+ *                 on its own; results are only complete with both.
  *
  * Rows whose visible key set is empty (time_dim_sizes[b] == 0 on an in-phase slot) are written
  * as zeros; the reference leaves 0/0 there and its caller ignores them (g4b/scheduler.py:142-148).
@@ -104,9 +108,11 @@ typedef struct g4b_attn_args {
 
 int g4b_attn_forward(const g4b_attn_args* args, void* stream);
 
-/* Bytes of workspace that let g4b_attn_forward split the keys of a decode-shaped launch
- * (R*Tq <= 16) over `num_workers` waves (0 = library default).  Returns 0 when the shape never
- * uses a workspace (prefill-shaped launches). */
+/* Bytes of workspace that let g4b_attn_forward split keys: for a decode-shaped launch (R*Tq <= 16)
+ * over `num_workers` waves (0 = library default); for a prefill shape that brings fewer workgroups
+ * per slot than the chip has compute units (chunked prefill, short prompts; sized by H, G, Tq, D
+ * only) over several workgroups per query tile.  Returns 0 when the shape never uses a workspace.
+ * Replaces the sizing of partial_o/l/m at g4b/models/gemma4e.py:43,819-821. */
 uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers);
 
 /* The library default for num_workers on the current build (a multiple of the CU count). */

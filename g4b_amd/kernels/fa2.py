@@ -55,7 +55,7 @@ def _private_workspace(q, nbytes: int):
     return ws
 
 
-def flash_attention(
+def _bind(
     q,
     k_cache,
     v_cache,
@@ -79,37 +79,8 @@ def flash_attention(
     workspace=None,
     num_workers: int = 0,
     kernel_mask: int = 0,
-    stream=None,
 ):
-    """``o[b, h, i] = softmax(scale * q[b, h, i] . K_b^T + mask) V_b`` for every in-phase slot ``b``.
-
-    Positional arguments and the first five keywords are the reference's (``fa2.py:634-652``):
-
-    * ``q``, ``o``: ``[B, H, Tq, D]`` (strided views allowed, unit stride in ``D``);
-      ``k_cache``, ``v_cache``: ``[B, G, KV_CTX, D]`` rings; ``time_dim_sizes``: ``[B]`` int32;
-      ``user_phase``: ``[B]`` uint8 -- slots with ``user_phase[b] != phase`` are skipped and their
-      rows of ``o`` stay untouched.
-    * ``partial_o/l/m``: the reference's split-KV scratch.  All three or none
-      (``ValueError`` otherwise, ``fa2.py:656-657``).  Passing them allows a decode launch to
-      split keys across workgroups, as in the reference; the partials themselves live in a
-      private workspace (or ``workspace=``) with this library's own layout, and the contents of
-      ``partial_*`` are left unspecified.
-    * ``use_grouped_query_tile``, ``warp_specialize``, ``is_hopper``, ``use_fp32_dot``: tuning
-      knobs of the Triton kernel; accepted and ignored (the GQA group is always packed and the
-      products always run on fp16/bf16 MFMA with fp32 accumulation).
-    * ``stage``: ``STAGE_CAUSAL`` or ``STAGE_FULL``.
-
-    Keyword-only extensions, with defaults that reproduce the reference:
-
-    * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
-      ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
-      ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
-      used for split partials instead of the private one; ``False`` = use none and never split); ``num_workers``; ``kernel_mask`` (profiling:
-      bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
-
-    Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
-    ignore (``g4b/models/gemma4e.py:593-607``).
-    """
+    """Validate the arguments like the reference and fill the C argument block (plus the objects it points into)."""
     assert isinstance(phase, int)  # fa2.py:653
     if (partial_o is None) != (partial_l is None) or (partial_o is None) != (partial_m is None):
         raise ValueError("partial_o, partial_l, and partial_m must be provided together")
@@ -192,5 +163,97 @@ def flash_attention(
         a.workspace = ws.data_ptr()
         a.workspace_bytes = int(ws.numel()) * int(ws.element_size()) if hasattr(ws, "numel") else int(ws.nbytes)
 
+    return a, (q, k_cache, v_cache, o, time_dim_sizes, user_phase, window_sizes, ws)
+
+
+def flash_attention(
+    q,
+    k_cache,
+    v_cache,
+    o,
+    time_dim_sizes,
+    user_phase,
+    ctx_window_size: int,
+    phase: int,
+    partial_o=None,
+    partial_l=None,
+    partial_m=None,
+    *,
+    use_grouped_query_tile: bool = True,
+    warp_specialize: bool = False,
+    is_hopper: bool = False,
+    use_fp32_dot: bool = False,
+    stage: int = STAGE_CAUSAL,
+    scale: float = 1.0,
+    query_window: int | None = None,
+    window_sizes=None,
+    workspace=None,
+    num_workers: int = 0,
+    kernel_mask: int = 0,
+    stream=None,
+):
+    """``o[b, h, i] = softmax(scale * q[b, h, i] . K_b^T + mask) V_b`` for every in-phase slot ``b``.
+
+    Positional arguments and the first five keywords are the reference's (``fa2.py:634-652``):
+
+    * ``q``, ``o``: ``[B, H, Tq, D]`` (strided views allowed, unit stride in ``D``);
+      ``k_cache``, ``v_cache``: ``[B, G, KV_CTX, D]`` rings; ``time_dim_sizes``: ``[B]`` int32;
+      ``user_phase``: ``[B]`` uint8 -- slots with ``user_phase[b] != phase`` are skipped and their
+      rows of ``o`` stay untouched.
+    * ``partial_o/l/m``: the reference's split-KV scratch.  All three or none
+      (``ValueError`` otherwise, ``fa2.py:656-657``).  Passing them allows a decode launch to
+      split keys across workgroups, as in the reference; the partials themselves live in a
+      private workspace (or ``workspace=``) with this library's own layout, and the contents of
+      ``partial_*`` are left unspecified.
+    * ``use_grouped_query_tile``, ``warp_specialize``, ``is_hopper``, ``use_fp32_dot``: tuning
+      knobs of the Triton kernel; accepted and ignored (the GQA group is always packed and the
+      products always run on fp16/bf16 MFMA with fp32 accumulation).
+    * ``stage``: ``STAGE_CAUSAL`` or ``STAGE_FULL``.
+
+    Keyword-only extensions, with defaults that reproduce the reference:
+
+    * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
+      ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
+      ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
+      used for split partials instead of the private one; ``False`` = use none and never split); ``num_workers``; ``kernel_mask`` (profiling:
+      bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
+
+    Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
+    ignore (``g4b/models/gemma4e.py:593-607``).
+    """
+    a, _keep = _bind(
+        q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, partial_o, partial_l, partial_m,
+        use_grouped_query_tile=use_grouped_query_tile, warp_specialize=warp_specialize, is_hopper=is_hopper,
+        use_fp32_dot=use_fp32_dot, stage=stage, scale=scale, query_window=query_window, window_sizes=window_sizes,
+        workspace=workspace, num_workers=num_workers, kernel_mask=kernel_mask,
+    )
+    lib = _native.load()
     _native.check(lib.g4b_attn_forward(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
     return None, None
+
+
+class AttentionPlan:
+    """A bound ``flash_attention`` call: arguments validated once, every ``launch()`` is the bare C call.
+
+    The engine records its steps into graphs (``g4b/lifecycle.py:29-53``), which is how the reference keeps
+    Python out of the decode loop; outside a graph this gives the same effect for callers whose tensors do not
+    move between steps (the caches, scratchpads and per-slot integer tensors of a serving engine never do).  The
+    plan holds references to the tensors it points into.
+    """
+
+    def __init__(self, args, keep):
+        self._args, self._keep = args, keep
+        self._lib = _native.load()
+        self._ref = C.byref(args)
+
+    def launch(self, stream=None) -> None:
+        rc = self._lib.g4b_attn_forward(self._ref, C.c_void_p(U.current_stream() if stream is None else int(stream)))
+        if rc:
+            _native.check(rc)
+
+
+def plan_flash_attention(*args, **kwargs) -> AttentionPlan:
+    """Same arguments as :func:`flash_attention` (without ``stream``); returns an :class:`AttentionPlan`."""
+    kwargs.pop("stream", None)
+    a, keep = _bind(*args, **kwargs)
+    return AttentionPlan(a, keep)

@@ -171,6 +171,24 @@ def test_prefill_workspace_too_small_is_refused(fa):
     assert_close(o.float().cpu().numpy(), oracle(q, k, v, [W], [1], W, 1, scale=1 / 16), what="caller workspace")
 
 
+def test_bound_plan_relaunches_with_new_device_data(fa):
+    """A plan binds pointers, not values: lengths and queries updated in place are seen by the next launch."""
+    B, H, G, D, W = 4, 8, 2, 256, 1024
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=17)
+    tds = i32([100, 1024, 1024 + 5, 7])
+    phase = u8([2, 2, 2, 2])
+    ws = torch.empty(fa.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device="cuda")
+    plan = fa.plan_flash_attention(q, k, v, o, tds, phase, W, 2, scale=1 / 16, workspace=ws)
+    plan.launch()
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), oracle(q, k, v, tds.tolist(), [2] * B, W, 2, scale=1 / 16), what="plan, first launch")
+    tds += 3
+    q.copy_(torch.roll(q, 1, dims=0))
+    plan.launch()
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), oracle(q, k, v, tds.tolist(), [2] * B, W, 2, scale=1 / 16), what="plan, second launch")
+
+
 def test_one_shot_causal_prefill_2048(fa):
     """BASELINE config 2: batch 1, seq 2048, 8 q heads / 2 kv heads, head dim 256, scale 1/16."""
     B, H, G, Tq, D = 1, 8, 2, 2048, 256

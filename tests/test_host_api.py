@@ -179,3 +179,16 @@ def test_tensor_protocol_accepts_g4b_style_tensors(native):
     assert U.strides_of(w) == list(t.stride()) == U.strides_of(t)
     assert U.float_dtype_code(w, "w") == U.float_dtype_code(t, "t") == native.DT_F16
     assert U.dtype_name(torch.zeros(1, dtype=torch.int32)) == "int32"
+
+
+def test_plan_validates_at_bind_time(native):
+    from g4b_amd.kernels.fa2 import PHASE_DECODE, plan_flash_attention
+
+    q, k, v, o, tds, ph = _decode_args()
+    plan = plan_flash_attention(q, k, v, o, tds, ph, 64, PHASE_DECODE, scale=0.5)
+    assert plan._args.B == 2 and plan._args.H == 8 and plan._args.KV_CTX == 64 and plan._args.scale == 0.5
+    with pytest.raises(ValueError):  # shape checks run when the plan is made (fa2.py:296)
+        plan_flash_attention(q[:, :7], k, v, o, tds, ph, 64, PHASE_DECODE)
+    bad = plan_flash_attention(q, k, v, o, tds, ph, 65, PHASE_DECODE)
+    with pytest.raises(ValueError, match="ctx_window_size"):  # value checks live in the library (fa2.py:298)
+        bad.launch(stream=0)

@@ -27,13 +27,12 @@
 // rescaled lazily.
 #include "common.hpp"
 #include "launch.hpp"
+#include "prefill_map.hpp"
 
 namespace g4b {
 
-constexpr int PF_BM = 128;     // query rows per workgroup
 constexpr int PF_BN = 64;      // keys per tile
 constexpr int PF_PD = 6;       // LDS operand fetches in flight (issued and retired in pairs)
-constexpr float PF_TAU = 8.f;  // log2 of the growth of a row maximum that triggers a rescale
 
 template <int D>
 struct PfSmem {
@@ -41,25 +40,6 @@ struct PfSmem {
     static constexpr int TILE = PF_BN * ROW;
     static constexpr int VSWZ = (D >= 256) ? 7 : 3;  // (V row & VSWZ) selects the 64-byte group swizzle
 };
-
-// Linear workgroup id -> (head, query tile rank) bookkeeping shared by the kernel and its launcher.
-struct PfMap {
-    int heads, nq, mode, grid;
-};
-__host__ __device__ inline PfMap pf_map(int heads, int nq) {
-    PfMap m;
-    m.heads = heads;
-    m.nq = nq;
-    if (heads <= 8 && 8 % heads == 0) {
-        const int share = 8 / heads;
-        m.mode = 1;
-        m.grid = 8 * ((nq + share - 1) / share);
-    } else {
-        m.mode = (heads % 8 == 0) ? 2 : 0;
-        m.grid = heads * nq;
-    }
-    return m;
-}
 
 template <int D, class T>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
@@ -80,10 +60,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     const int n32 = lane & 31, h2 = lane >> 5;
     const int R = p.R, Tq = p.Tq, KV_CTX = p.KV_CTX;
     const int TOKB = PF_BM / R;
-    // Work item of this workgroup: (kv head of a slot, query tile).  Workgroups are handed to the 8 XCDs round-robin
-    // by their linear id and every XCD has an L2 of its own, so the ids are mapped such that an XCD walks the K/V of
-    // as few heads as possible, its workgroups start at the same key and advance together (one fetch from memory
-    // serves the XCD), the heaviest (latest) query tiles start first, and the XCDs get equal shares.
     // The work list is built from the slots that are in phase, so a launch with few of them (one prefill chunk in a
     // batch of decoding slots) can split every item's keys over several workgroups and still fill the chip.
     __shared__ int sh_scan[8];
@@ -94,19 +70,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     const PfMap map = pf_map(n_active * p.G * nsplit, (Tq + TOKB - 1) / TOKB);
     if ((int)blockIdx.x >= map.grid) return;
     int head, rank;
-    {
-        const int f = blockIdx.x, x = f & 7, j = f >> 3;
-        if (map.mode == 1) {  // heads divide 8: 8 / heads XCDs share a head and take its query tiles in turn
-            head = x % map.heads;
-            rank = j * (8 / map.heads) + x / map.heads;
-        } else if (map.mode == 2) {  // 8 divides heads: every XCD owns heads / 8 heads
-            head = (j % (map.heads / 8)) * 8 + x;
-            rank = j / (map.heads / 8);
-        } else {
-            head = f % map.heads;
-            rank = f / map.heads;
-        }
-    }
+    pf_item(map, blockIdx.x, head, rank);
     if (rank >= map.nq) return;
     const int qtile = map.nq - 1 - rank;
     const int split = head % nsplit, g = (head / nsplit) % p.G, a_idx = head / (nsplit * p.G);
@@ -545,12 +509,8 @@ __global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) 
 template <int D, class T>
 static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     const int TOKB = PF_BM / p.R;
-    // The grid is sized for the worst case over the number of slots that turn out to be in phase; the kernel reads
-    // that number on the device and surplus workgroups leave at once.
-    const int nq = (p.Tq + TOKB - 1) / TOKB;
     const int slots = p.part_o ? p.split_slots : 1;
-    int blocks = 0;
-    for (int n = 1; n <= p.B; ++n) blocks = max(blocks, pf_map(n * p.G * prefill_splits(slots, n), nq).grid);
+    const int blocks = prefill_grid(p);
     dim3 grid(blocks);
     const int smem = 4 * PfSmem<D>::TILE;
     static bool attr_set = false;

@@ -255,9 +255,10 @@ G4B_DEV SlotInfo slot_info(const AttnParams& p, int b) {
 }
 
 // Number of slots whose phase matches the launch (n_active) and the index of the a-th of them (-1 when a is out of
-// range).  Every thread of a 256-thread workgroup must call it; sh is workgroup-shared scratch of at least 5 ints.
-// Call it with a < 0 to count only.
-G4B_DEV int nth_active_slot(const AttnParams& p, int a, int& n_active, int* sh) {
+// range).  Every thread of a workgroup of NWAVES waves must call it; sh is workgroup-shared scratch of at least
+// NWAVES + 1 ints.  Call it with a < 0 to count only.
+template <int NWAVES>
+G4B_DEV int nth_active_slot_t(const AttnParams& p, int a, int& n_active, int* sh) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (p.B <= 64) {  // one ballot per wave answers both questions, no exchange between waves
         const bool act = lane < p.B && p.phase_arr[(int64_t)lane * p.ph_s] == (uint8_t)p.phase;
@@ -268,7 +269,7 @@ G4B_DEV int nth_active_slot(const AttnParams& p, int a, int& n_active, int* sh) 
         return __ffsll((long long)hit) - 1;
     }
     int base = 0;
-    for (int c0 = 0; c0 < p.B; c0 += 256) {
+    for (int c0 = 0; c0 < p.B; c0 += 64 * NWAVES) {
         const int b = c0 + tid;
         const bool act = b < p.B && p.phase_arr[(int64_t)b * p.ph_s] == (uint8_t)p.phase;
         const unsigned long long m = __ballot(act);
@@ -276,15 +277,19 @@ G4B_DEV int nth_active_slot(const AttnParams& p, int a, int& n_active, int* sh) 
         __syncthreads();
         int before = base;
         for (int w = 0; w < wave; ++w) before += sh[w];
-        const int total = sh[0] + sh[1] + sh[2] + sh[3];
+        int total = 0;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) total += sh[w];
         const int rank = before + __popcll(m & ((1ull << lane) - 1ull));
-        if (act && rank == a) sh[4] = b;
+        if (act && rank == a) sh[NWAVES] = b;
         base += total;
         __syncthreads();
     }
     n_active = base;
-    return (a >= 0 && a < base) ? sh[4] : -1;
+    return (a >= 0 && a < base) ? sh[NWAVES] : -1;
 }
+G4B_DEV int nth_active_slot(const AttnParams& p, int a, int& n_active, int* sh) { return nth_active_slot_t<4>(p, a, n_active, sh); }
+
 
 // Key splits per active slot of a prefill-shaped launch: the partial buffers hold split_slots (slot, split) pairs.
 __host__ __device__ inline int prefill_splits(int split_slots, int n_active) {

@@ -1,0 +1,60 @@
+// Work-item bookkeeping shared by the prefill kernels and their launcher.
+#pragma once
+#include "common.hpp"
+
+namespace g4b {
+
+constexpr int PF_BM = 128;     // query rows per workgroup
+constexpr float PF_TAU = 8.f;  // log2 of the growth of a row maximum that triggers a rescale
+
+// Linear workgroup id -> (head, query tile rank).  "Heads" are (active slot, kv head, key split) triples.  Workgroups
+// are handed to the 8 XCDs round-robin by their linear id and every XCD has an L2 of its own, so the ids are mapped
+// such that an XCD walks the K/V of as few heads as possible, its workgroups start at the same key and advance
+// together (one fetch from memory serves the XCD), the heaviest (latest) query tiles start first, and the XCDs get
+// equal shares.
+struct PfMap {
+    int heads, nq, mode, grid;
+};
+__host__ __device__ inline PfMap pf_map(int heads, int nq) {
+    PfMap m;
+    m.heads = heads;
+    m.nq = nq;
+    if (heads <= 8 && 8 % heads == 0) {
+        const int share = 8 / heads;
+        m.mode = 1;
+        m.grid = 8 * ((nq + share - 1) / share);
+    } else {
+        m.mode = (heads % 8 == 0) ? 2 : 0;
+        m.grid = heads * nq;
+    }
+    return m;
+}
+__host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int& rank) {
+    const int x = f & 7, j = f >> 3;
+    if (map.mode == 1) {  // heads divide 8: 8 / heads XCDs share a head and take its query tiles in turn
+        head = x % map.heads;
+        rank = j * (8 / map.heads) + x / map.heads;
+    } else if (map.mode == 2) {  // 8 divides heads: every XCD owns heads / 8 heads
+        head = (j % (map.heads / 8)) * 8 + x;
+        rank = j / (map.heads / 8);
+    } else {
+        head = f % map.heads;
+        rank = f / map.heads;
+    }
+}
+
+// Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on
+// the device and surplus workgroups leave at once.
+inline int prefill_grid(const AttnParams& p) {
+    const int tokb = PF_BM / p.R;
+    const int nq = (p.Tq + tokb - 1) / tokb;
+    const int slots = p.part_o ? p.split_slots : 1;
+    int blocks = 0;
+    for (int n = 1; n <= p.B; ++n) {
+        const int g = pf_map(n * p.G * prefill_splits(slots, n), nq).grid;
+        blocks = g > blocks ? g : blocks;
+    }
+    return blocks;
+}
+
+}  // namespace g4b

@@ -128,8 +128,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 #pragma unroll
         for (int i = 0; i < CHUNKS; ++i) {
             const int row = st_row(i);
-            k_const[i] = (uint32_t)row * SM::ROW + (uint32_t)k_piece(row) * 16u;
-            v_const[i] = (uint32_t)row * SM::ROW + (uint32_t)v_piece(row) * 16u;
+            // chunk i is issued with instruction offset (i % 4) KiB, which moves source and destination alike
+            k_const[i] = (uint32_t)row * SM::ROW + (uint32_t)k_piece(row) * 16u - (uint32_t)(i & 3) * 1024u;
+            v_const[i] = (uint32_t)row * SM::ROW + (uint32_t)v_piece(row) * 16u - (uint32_t)(i & 3) * 1024u;
         }
         auto plain_row0 = [&](int kt) -> int {  // ring row of the tile's first key, or -1
             const int jb = kt * PF_BN;
@@ -138,7 +139,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             r0 = (r0 >= KV_CTX) ? r0 - KV_CTX : r0;
             return (r0 + PF_BN <= KV_CTX) ? r0 : -1;
         };
-        // Source of K or V tile kt as scalar base + per-lane byte offsets.
+        // Source of K or V tile kt as scalar base + per-lane byte offsets (the instruction offset of chunk i comes on
+        // top: on the general path the base is lowered by 3 KiB so that the lane offsets stay non-negative).
         auto tile_src = [&](int kt, bool is_v, const char*& src, uint32_t(&ofs)[CHUNKS]) {
             const int r0 = plain_row0(kt);
             const char* base = is_v ? vbase : kbase;
@@ -147,22 +149,31 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
 #pragma unroll
                 for (int i = 0; i < CHUNKS; ++i) ofs[i] = is_v ? v_const[i] : k_const[i];
             } else {
-                src = base;
+                src = base - 3072;
 #pragma unroll
                 for (int i = 0; i < CHUNKS; ++i) {
                     const int row = st_row(i);
-                    ofs[i] = key_off(kt * PF_BN + row) + (uint32_t)(is_v ? v_piece(row) : k_piece(row)) * 16u;
+                    ofs[i] = key_off(kt * PF_BN + row) + (uint32_t)(is_v ? v_piece(row) : k_piece(row)) * 16u + 3072u -
+                             (uint32_t)(i & 3) * 1024u;
                 }
             }
         };
         const uint32_t wave_chunk0 = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (CHUNKS * 1024);
+        // chunk i of a tile: four chunks share one M0 base
+        auto dma_chunk = [&](int i, const char* src, const uint32_t(&ofs)[CHUNKS], uint32_t dst) {
+            if ((i & 3) == 0) dma_set_base(dst + i * 1024);
+            if ((i & 3) == 0) dma16_to_lds_at<0>(src, ofs[i]);
+            if ((i & 3) == 1) dma16_to_lds_at<1024>(src, ofs[i]);
+            if ((i & 3) == 2) dma16_to_lds_at<2048>(src, ofs[i]);
+            if ((i & 3) == 3) dma16_to_lds_at<3072>(src, ofs[i]);
+        };
         auto stage_whole_tile = [&](int kt, bool is_v, int stage) {  // prologue only: all chunks at once
             const char* src;
             uint32_t ofs[CHUNKS];
             tile_src(kt, is_v, src, ofs);
             const uint32_t dst = lds0 + (is_v ? 2 * SM::TILE : 0) + stage * SM::TILE + wave_chunk0;
 #pragma unroll
-            for (int i = 0; i < CHUNKS; ++i) dma16_to_lds(src, ofs[i], dst + i * 1024);
+            for (int i = 0; i < CHUNKS; ++i) dma_chunk(i, src, ofs, dst);
         };
 
         // ---- operand read offsets (bytes from the start of a stage pair) ----------------------------------------
@@ -316,9 +327,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                 // One direct load per pair: K(kt+2) first (its stage was released by the barrier that ended the
                 // previous tile and it is needed first), then V(kt+1).  Issued this early, the loads have the rest
                 // of the tile to land before the closing barrier waits for them.
-                if (idx / 2 < CHUNKS) dma16_to_lds(ksrc, kofs[idx / 2], kdst + (idx / 2) * 1024);
+                if (idx / 2 < CHUNKS) dma_chunk(idx / 2, ksrc, kofs, kdst);
                 if (idx / 2 >= CHUNKS && idx / 2 < 2 * CHUNKS)
-                    dma16_to_lds(vsrc, vofs[idx / 2 - CHUNKS], vdst + (idx / 2 - CHUNKS) * 1024);
+                    dma_chunk(idx / 2 - CHUNKS, vsrc, vofs, vdst);
             };
 #pragma unroll
             for (int idx = 0; idx < N1; idx += 2) qk_pair(idx);

@@ -167,10 +167,15 @@ G4B_DEV u4 lds_read16(uint32_t lds_addr, int imm) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(imm));
     return v;
 }
-// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16 * l (M0 carries the base).
-// Source address = scalar base + per-lane 32-bit offset.  Completion is tracked by vmcnt.
-G4B_DEV void dma16_to_lds(const void* sbase, uint32_t voff, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
+// 16 bytes per lane from global memory straight into LDS: lane l lands at M0 + IMM + 16 * l and comes from
+// scalar base + per-lane 32-bit offset + IMM (the instruction offset moves both ends; 0 <= IMM < 4096).  Completion
+// is tracked by vmcnt.  dma_set_base loads M0; one base serves the loads that follow it until the next dma_set_base
+// (nothing else in these kernels touches M0).
+G4B_DEV void dma_set_base(uint32_t lds_base) { asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(lds_base) : "m0"); }
+template <int IMM>
+G4B_DEV void dma16_to_lds_at(const void* sbase, uint32_t voff) {
+    static_assert(IMM >= 0 && IMM < 4096, "13-bit signed instruction offset");
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(voff), "s"(sbase), "n"(IMM) : "memory");
 }
 G4B_DEV void vm_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

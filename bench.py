@@ -39,8 +39,8 @@ FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # Counters cannot be read from inside the timed run, so the figures are carried here; a workload without a
 # counter run reports null.
 PMC_TRAFFIC_KIB = {
-    "decode_batched_b64": {"fetch": 579346.4, "write": 4544.8},
-    "prefill_causal_8192": {"fetch": 186678.2, "write": 32768.0},
+    "decode_batched_b64": {"fetch": 579346.1, "write": 4544.8},
+    "prefill_causal_8192": {"fetch": 82093.4, "write": 32768.0},
 }
 PMC_SCALE = {"fetch": 2.000, "write": 1.000}
 

@@ -95,12 +95,59 @@ class AdvanceArgs(C.Structure):
     ]
 
 
+class RopeArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p),
+        ("k", C.c_void_p),
+        ("rope_freqs", C.c_void_p),
+        ("time_dim_offsets", C.c_void_p),
+        ("q_rsos", C.c_void_p),
+        ("k_rsos", C.c_void_p),
+        ("q_rmsnorm_w", C.c_void_p),
+        ("k_rmsnorm_w", C.c_void_p),
+        ("v", C.c_void_p),
+        ("v_rsos", C.c_void_p),
+        ("k_cache", C.c_void_p),
+        ("v_cache", C.c_void_p),
+        ("user_phase", C.c_void_p),
+        ("q_stride", C.c_int64 * 4),
+        ("k_stride", C.c_int64 * 4),
+        ("v_stride", C.c_int64 * 4),
+        ("q_rsos_stride", C.c_int64 * 3),
+        ("k_rsos_stride", C.c_int64 * 3),
+        ("v_rsos_stride", C.c_int64 * 3),
+        ("rope_freqs_stride", C.c_int64),
+        ("q_rmsnorm_w_stride", C.c_int64),
+        ("k_rmsnorm_w_stride", C.c_int64),
+        ("time_dim_offsets_stride", C.c_int64),
+        ("user_phase_stride", C.c_int64),
+        ("k_cache_stride_b", C.c_int64),
+        ("v_cache_stride_b", C.c_int64),
+        ("q_dtype", C.c_int32),
+        ("k_dtype", C.c_int32),
+        ("v_dtype", C.c_int32),
+        ("cache_dtype", C.c_int32),
+        ("B", C.c_int32),
+        ("H", C.c_int32),
+        ("G", C.c_int32),
+        ("t", C.c_int32),
+        ("D", C.c_int32),
+        ("Dv", C.c_int32),
+        ("T", C.c_int32),
+        ("phase", C.c_int32),
+        ("k_writeback", C.c_int32),
+        ("rmsnorm_eps", C.c_float),
+    ]
+
+
 EXPORTS = {
     "g4b_attn_forward": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p]),
     "g4b_attn_workspace_bytes": (C.c_uint64, [C.c_int32] * 6),
     "g4b_attn_default_workers": (C.c_int32, []),
     "g4b_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), C.c_void_p]),
     "g4b_advance_decode_state": (C.c_int, [C.POINTER(AdvanceArgs), C.c_void_p]),
+    "g4b_rope": (C.c_int, [C.POINTER(RopeArgs), C.c_void_p]),
+    "g4b_rope_frequencies": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_float, C.c_void_p]),
     "g4b_last_error": (C.c_char_p, []),
     "g4b_abi_version": (C.c_int32, []),
 }

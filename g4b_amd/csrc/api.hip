@@ -230,4 +230,101 @@ int g4b_advance_decode_state(const g4b_advance_args* a, void* stream) {
     return G4B_OK;
 }
 
+int g4b_rope(const g4b_rope_args* a, void* stream) {
+    if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
+    if (!a->q || !a->k || !a->rope_freqs || !a->time_dim_offsets || !a->q_rsos || !a->k_rsos || !a->q_rmsnorm_w || !a->k_rmsnorm_w)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "q, k, rope_freqs, time_dim_offsets, q/k_rsos and q/k_rmsnorm_w must be non-NULL");
+    if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype)) return fail(G4B_ERR_INVALID_ARGUMENT, "q/k dtype must be f16, bf16 or f32");
+    if (a->B < 1 || a->H < 1 || a->G < 1 || a->t < 1 || a->D < 1) return fail(G4B_ERR_INVALID_ARGUMENT, "B, H, G, t, D must be positive");
+    if (a->D % 16 || a->D > 4096) return fail(G4B_ERR_UNSUPPORTED, "D must be a multiple of 16 and at most 4096 (got %d)", a->D);
+    if (a->B > 65535) return fail(G4B_ERR_UNSUPPORTED, "B must be <= 65535");
+    if (a->q_stride[3] != 1 || a->k_stride[3] != 1) return fail(G4B_ERR_INVALID_ARGUMENT, "q and k must have unit stride in the head dimension");
+    for (int i = 0; i < 3; ++i)
+        if (a->q_stride[i] % 8 || a->k_stride[i] % 8) return fail(G4B_ERR_INVALID_ARGUMENT, "q/k strides must be multiples of 8 elements");
+    if (!aligned16(a->q) || !aligned16(a->k)) return fail(G4B_ERR_INVALID_ARGUMENT, "q and k must be 16-byte aligned");
+    if (!std::isfinite(a->rmsnorm_eps)) return fail(G4B_ERR_INVALID_ARGUMENT, "rmsnorm_eps must be finite");
+    if (a->k_cache) {
+        if (!dtype_ok(a->cache_dtype)) return fail(G4B_ERR_INVALID_ARGUMENT, "cache dtype must be f16, bf16 or f32");
+        if (a->T < 1 || a->t > a->T) return fail(G4B_ERR_INVALID_ARGUMENT, "t (%d) must not exceed the ring length T (%d)", a->t, a->T);
+        if (a->phase < 0 || a->phase > 255) return fail(G4B_ERR_INVALID_ARGUMENT, "phase must fit uint8");
+        if (a->k_cache_stride_b < (int64_t)a->G * a->T * a->D || a->k_cache_stride_b % 8)
+            return fail(G4B_ERR_INVALID_ARGUMENT, "k_cache slot stride must be >= G*T*D and a multiple of 8 elements");
+        if (!aligned16(a->k_cache)) return fail(G4B_ERR_INVALID_ARGUMENT, "k_cache must be 16-byte aligned");
+        if ((a->v != nullptr) != (a->v_cache != nullptr)) return fail(G4B_ERR_INVALID_ARGUMENT, "v and v_cache go together");
+        if (a->v) {
+            if (!dtype_ok(a->v_dtype)) return fail(G4B_ERR_INVALID_ARGUMENT, "v dtype must be f16, bf16 or f32");
+            if (a->Dv < 1 || a->Dv % 8) return fail(G4B_ERR_UNSUPPORTED, "Dv must be a positive multiple of 8");
+            if (a->v_stride[3] != 1) return fail(G4B_ERR_INVALID_ARGUMENT, "v must have unit stride in the head dimension");
+            for (int i = 0; i < 3; ++i)
+                if (a->v_stride[i] % 8) return fail(G4B_ERR_INVALID_ARGUMENT, "v strides must be multiples of 8 elements");
+            if (a->v_cache_stride_b < (int64_t)a->G * a->T * a->Dv || a->v_cache_stride_b % 8)
+                return fail(G4B_ERR_INVALID_ARGUMENT, "v_cache slot stride must be >= G*T*Dv and a multiple of 8 elements");
+            if (!aligned16(a->v) || !aligned16(a->v_cache)) return fail(G4B_ERR_INVALID_ARGUMENT, "v and v_cache must be 16-byte aligned");
+        }
+    } else if (a->v || a->v_cache) {
+        return fail(G4B_ERR_INVALID_ARGUMENT, "v / v_cache need k_cache: the append is fused as a whole");
+    }
+
+    g4b::RopeParams p{};
+    p.q = a->q;
+    p.k = a->k;
+    p.freqs = a->rope_freqs;
+    p.offsets = a->time_dim_offsets;
+    p.q_rsos = a->q_rsos;
+    p.k_rsos = a->k_rsos;
+    p.q_w = a->q_rmsnorm_w;
+    p.k_w = a->k_rmsnorm_w;
+    p.v = a->v;
+    p.v_rsos = a->v_rsos;
+    p.k_cache = a->k_cache;
+    p.v_cache = a->v_cache;
+    p.phase_arr = a->user_phase;
+    for (int i = 0; i < 4; ++i) {
+        p.q_s[i] = a->q_stride[i];
+        p.k_s[i] = a->k_stride[i];
+        p.v_s[i] = a->v_stride[i];
+    }
+    for (int i = 0; i < 3; ++i) {
+        p.q_rsos_s[i] = a->q_rsos_stride[i];
+        p.k_rsos_s[i] = a->k_rsos_stride[i];
+        p.v_rsos_s[i] = a->v_rsos_stride[i];
+    }
+    p.freqs_s = a->rope_freqs_stride;
+    p.q_w_s = a->q_rmsnorm_w_stride;
+    p.k_w_s = a->k_rmsnorm_w_stride;
+    p.off_s = a->time_dim_offsets_stride;
+    p.ph_s = a->user_phase_stride;
+    p.k_cache_sb = a->k_cache_stride_b;
+    p.v_cache_sb = a->v_cache_stride_b;
+    p.q_dt = a->q_dtype;
+    p.k_dt = a->k_dtype;
+    p.v_dt = a->v_dtype;
+    p.cache_dt = a->cache_dtype;
+    p.B = a->B;
+    p.H = a->H;
+    p.G = a->G;
+    p.t = a->t;
+    p.D = a->D;
+    p.Dv = a->Dv;
+    p.T = a->T;
+    p.phase = a->phase;
+    p.k_writeback = a->k_writeback;
+    p.eps = a->rmsnorm_eps;
+    hipError_t e = g4b::launch_rope(p, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "rope launch failed: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
+int g4b_rope_frequencies(float* out, const float* freq_scalars, int32_t n, int64_t out_stride, int64_t freq_scalars_stride,
+                         float freq_base, void* stream) {
+    if (!out || n < 1) return fail(G4B_ERR_INVALID_ARGUMENT, "out must be non-NULL and n positive");
+    if (!(freq_base > 0.f) || !std::isfinite(freq_base)) return fail(G4B_ERR_INVALID_ARGUMENT, "freq_base must be positive and finite");
+    // the reference folds log2(freq_base) on the host in double precision (rope.py:280)
+    const float log2_base = (float)std::log2((double)freq_base);
+    hipError_t e = g4b::launch_rope_frequencies(out, freq_scalars, n, out_stride, freq_scalars_stride, log2_base,
+                                                static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "rope frequency launch failed: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
 }  // extern "C"

@@ -40,4 +40,31 @@ struct AdvanceParams {
 };
 hipError_t launch_advance_decode_state(const AdvanceParams& p, hipStream_t stream);
 
+struct RopeParams {
+    void* q;
+    void* k;
+    const float* freqs;
+    const int32_t* offsets;
+    const float* q_rsos;
+    const float* k_rsos;
+    const float* q_w;
+    const float* k_w;
+    const void* v;          // optional: fused append
+    const float* v_rsos;    // optional
+    void* k_cache;          // optional: fused append
+    void* v_cache;
+    const uint8_t* phase_arr;  // optional
+    int64_t q_s[4], k_s[4], v_s[4];
+    int64_t q_rsos_s[3], k_rsos_s[3], v_rsos_s[3];
+    int64_t freqs_s, q_w_s, k_w_s, off_s, ph_s;
+    int64_t k_cache_sb, v_cache_sb;
+    int32_t q_dt, k_dt, v_dt, cache_dt;
+    int32_t B, H, G, t, D, Dv, T;
+    int32_t phase, k_writeback;
+    float eps;
+};
+hipError_t launch_rope(const RopeParams& p, hipStream_t stream);
+hipError_t launch_rope_frequencies(float* out, const float* scalars, int n, int64_t out_s, int64_t sc_s, float log2_base,
+                                   hipStream_t stream);
+
 }  // namespace g4b

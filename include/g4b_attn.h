@@ -167,6 +167,67 @@ typedef struct g4b_advance_args {
 
 int g4b_advance_decode_state(const g4b_advance_args* args, void* stream);
 
+/*
+ * g4b_rope replaces apply_rope() (g4b/kernels/rope.py:123-243): for x in (q, k), in place,
+ *   x[b,h,t,:] <- rope(x[b,h,t,:] * rsqrt(x_rsos[b,h,t] / D + eps) * x_rmsnorm_w[:], theta[b,t,:])
+ *   theta[b,t,j] = (time_dim_offsets[b] + t) * rope_freqs[j]  (fp32),  j < D/2
+ *   rope(x)[j] = cos*x[j] - sin*x[j + D/2];   rope(x)[j + D/2] = cos*x[j + D/2] + sin*x[j]
+ * on every slot (the reference's kernel has no phase skip).  With k_cache non-NULL the same launch also
+ * does the two add_kv_to_cache() calls that follow it in the engine (g4b/models/gemma4e.py:575-590):
+ *   k_cache[b, g, (t + time_dim_offsets[b]) % T, :] = rotated k[b,g,t,:]
+ *   v_cache[b, g, (t + time_dim_offsets[b]) % T, :] = v[b,g,t,:] * (v_rsos ? rsqrt(v_rsos[b,g,t] / Dv + eps) : 1)
+ * for slots with user_phase[b] == phase (all slots when user_phase is NULL); the rotated k is then written
+ * back to k only if k_writeback != 0 (nothing in the engine reads it after the append).
+ *   q [B,H,t,D], k [B,G,t,D], v [B,G,t,Dv]: strided, last stride 1, f16/bf16/f32; rope_freqs [D/2] f32;
+ *   time_dim_offsets [B] int32; *_rsos [B,heads,t] f32 strided; *_rmsnorm_w [D] f32; caches [B,G,T,D(v)]
+ *   contiguous inside a slot, f16/bf16/f32; D and Dv multiples of 16; t <= T.
+ */
+typedef struct g4b_rope_args {
+    void* q;
+    void* k;
+    const float* rope_freqs;
+    const int32_t* time_dim_offsets;
+    const float* q_rsos;
+    const float* k_rsos;
+    const float* q_rmsnorm_w;
+    const float* k_rmsnorm_w;
+    const void* v;
+    const float* v_rsos;
+    void* k_cache;
+    void* v_cache;
+    const uint8_t* user_phase;
+    int64_t q_stride[4];
+    int64_t k_stride[4];
+    int64_t v_stride[4];
+    int64_t q_rsos_stride[3];
+    int64_t k_rsos_stride[3];
+    int64_t v_rsos_stride[3];
+    int64_t rope_freqs_stride;
+    int64_t q_rmsnorm_w_stride;
+    int64_t k_rmsnorm_w_stride;
+    int64_t time_dim_offsets_stride;
+    int64_t user_phase_stride;
+    int64_t k_cache_stride_b;
+    int64_t v_cache_stride_b;
+    int32_t q_dtype;
+    int32_t k_dtype;
+    int32_t v_dtype;
+    int32_t cache_dtype;
+    int32_t B, H, G, t, D, Dv, T;
+    int32_t phase;
+    int32_t k_writeback;
+    float rmsnorm_eps;
+} g4b_rope_args;
+
+int g4b_rope(const g4b_rope_args* args, void* stream);
+
+/*
+ * g4b_rope_frequencies replaces populate_rope_frequencies() (g4b/kernels/rope.py:262-293), run once at load:
+ *   out[j] = 1 / freq_base ** (j / n)  [/ freq_scalars[j]],  j < n;  out and freq_scalars are f32 device arrays.
+ */
+int g4b_rope_frequencies(float* out, const float* freq_scalars, int32_t n, int64_t out_stride,
+                         int64_t freq_scalars_stride, float freq_base, void* stream);
+
 /* Message of the calling thread's last failed call ("" if none). */
 const char* g4b_last_error(void);
 

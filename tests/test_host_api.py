@@ -49,6 +49,7 @@ def test_struct_layouts_match_the_header(native):
         ("g4b_attn_args", native.AttnArgs),
         ("g4b_kv_append_args", native.KvAppendArgs),
         ("g4b_advance_args", native.AdvanceArgs),
+        ("g4b_rope_args", native.RopeArgs),
     ):
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), header, re.S).group(1)
         fields = []

@@ -306,6 +306,46 @@ class MixedStep(Workload):
         raise NotImplementedError
 
 
+class RopeAppend(Workload):
+    """The step in front of the attention of a prefill chunk: q/k RMSNorm + rotary embedding on fp32 scratchpads in
+    engine layout ([B, t, heads, D] viewed as [B, heads, t, D]) with rotated K and normalised V written to fp16 rings,
+    one launch.  Algorithmic bytes: q read and written, k and v read, both new cache rows written."""
+
+    bound = "hbm"
+
+    def __init__(self, device, t=8192, seed=0):
+        import torch
+
+        from g4b_amd.kernels import rope
+
+        self.rope = rope
+        self.name = f"rope_append_t{t}"
+        self.t = t
+        g = torch.Generator(device=device).manual_seed(seed)
+        self.q = torch.randn(1, t, H, D, generator=g, device=device).permute(0, 2, 1, 3)
+        self.k = torch.randn(1, t, G, D, generator=g, device=device).permute(0, 2, 1, 3)
+        self.v = torch.randn(1, t, G, D, generator=g, device=device).permute(0, 2, 1, 3)
+        self.q_rsos, self.k_rsos, self.v_rsos = (torch.full(x.shape[:3], float(D), device=device) for x in (self.q, self.k, self.v))
+        self.freqs = torch.empty(D // 2, device=device)
+        rope.populate_rope_frequencies(self.freqs, None, 1e6)
+        self.qw = torch.ones(D, device=device)
+        self.kw = torch.ones(D, device=device)
+        self.kc = torch.zeros(1, G, t, D, dtype=torch.float16, device=device)
+        self.vc = torch.zeros(1, G, t, D, dtype=torch.float16, device=device)
+        self.offs = torch.zeros(1, dtype=torch.int32, device=device)
+        self.bytes = t * D * (2 * H * 4 + 2 * G * 4 + 2 * G * 2)
+        self.flops = 0
+        self.units = self.bytes
+
+    def launch(self, i=0, kernel_mask=0):
+        # rsos = D and unit weights: the normalisation is the identity, so repeated in-place launches stay bounded
+        self.rope.apply_rope_and_append(self.q, self.k, self.v, self.freqs, self.offs, self.q_rsos, self.k_rsos, self.v_rsos,
+                                        self.qw, self.kw, 0.0, self.kc, self.vc)
+
+    def cpu_sample(self):
+        raise NotImplementedError
+
+
 WORKLOADS = {
     "decode_batched": lambda dev: BatchedDecode(dev),
     "decode_single": lambda dev: SingleDecode(dev),
@@ -313,6 +353,7 @@ WORKLOADS = {
     "prefill_causal_8192": lambda dev: Prefill(dev, 8192),
     "prefill_swa_8192": lambda dev: Prefill(dev, 8192, query_window=512),
     "mixed_step": lambda dev: MixedStep(dev),
+    "rope_append": lambda dev: RopeAppend(dev),
 }
 
 

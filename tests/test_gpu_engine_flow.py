@@ -160,3 +160,79 @@ def test_prefill_chunks_then_decode(gpu_device, W, context_len):
         assert tds.tolist() == [ctx[b] + 1 if b in decoding else 0 for b in range(B)]
         assert offsets.tolist() == [ctx[b] if b in decoding else 0 for b in range(B)]
         assert inp[0].tolist() == [b + 100 * step if b in decoding else 0 for b in range(B)]
+
+
+def test_rope_append_attention_by_absolute_position(gpu_device):
+    """gemma4e.py:564-607 with the rope, both appends and the attention of a layer: a stream fed as two prefill chunks
+    and three decode steps must give, at every new position, what the whole stream gives when it is normalised and
+    rotated by absolute position on the CPU and attended in one piece."""
+    from g4b_amd.kernels.advance_decode_state import advance_decode_state
+    from g4b_amd.kernels.fa2 import PHASE_DECODE, PHASE_PREFILL, flash_attention
+    from g4b_amd.kernels.rope import apply_rope_and_append
+    from oracle import rope_ref as rr
+
+    dev = gpu_device
+    B, H, G, D, t = 2, 8, 2, 256, 48  # slot 1 is never allocated
+    W = 4096
+    T = W + t - 1
+    eps, scale = 1e-6, 1.0
+    rng = np.random.default_rng(7)
+    n_total = 2 * t + 3
+    q_all = rng.standard_normal((H, n_total, D)).astype(np.float32)
+    k_all = rng.standard_normal((G, n_total, D)).astype(np.float32)
+    v_all = rng.standard_normal((G, n_total, D)).astype(np.float32)
+    freqs = rr.populate_rope_frequencies_ref(D // 2, 1e6).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    # whole stream on the CPU: positions 0 .. n_total - 1
+    q_rot, k_rot = rr.apply_rope_ref(q_all[None], k_all[None], freqs, np.array([0]), (q_all * q_all).sum(-1)[None],
+                                     (k_all * k_all).sum(-1)[None], qw, kw, eps)
+    v_n = v_all / np.sqrt((v_all * v_all).mean(-1, keepdims=True) + eps)
+    k16, v16 = k_rot[0].astype(np.float16), v_n.astype(np.float16)
+
+    q_pad = torch.zeros(B, t, H, D, device=dev)
+    k_pad = torch.zeros(B, t, G, D, device=dev)
+    v_pad = torch.zeros(B, t, G, D, device=dev)
+    o_pad = torch.zeros(B, t, H, D, device=dev)
+    q_rs, k_rs, v_rs = (torch.ones(B, t, n, device=dev) for n in (H, G, G))
+    k_cache = torch.zeros(B, G, T, D, device=dev, dtype=torch.float16)
+    v_cache = torch.zeros(B, G, T, D, device=dev, dtype=torch.float16)
+    freqs_d, qw_d, kw_d = (torch.from_numpy(x).to(dev) for x in (freqs, qw, kw))
+    offsets = torch.zeros(B, dtype=torch.int32, device=dev)
+    tds = torch.zeros(B, dtype=torch.int32, device=dev)
+    phase = torch.zeros(B, dtype=torch.uint8, device=dev)
+
+    def view(x, n):
+        return x[:, :n].permute(0, 2, 1, 3)
+
+    def step(lo, n, phase_id):
+        q_pad[0, :n] = torch.from_numpy(q_all[:, lo : lo + n].transpose(1, 0, 2)).to(dev)
+        k_pad[0, :n] = torch.from_numpy(k_all[:, lo : lo + n].transpose(1, 0, 2)).to(dev)
+        v_pad[0, :n] = torch.from_numpy(v_all[:, lo : lo + n].transpose(1, 0, 2)).to(dev)
+        for rs, x in ((q_rs, q_pad), (k_rs, k_pad), (v_rs, v_pad)):
+            rs[:, :n] = (x[:, :n] ** 2).sum(-1)
+        apply_rope_and_append(view(q_pad, n), view(k_pad, n), view(v_pad, n), freqs_d, offsets, q_rs[:, :n].permute(0, 2, 1),
+                              k_rs[:, :n].permute(0, 2, 1), v_rs[:, :n].permute(0, 2, 1), qw_d, kw_d, eps, k_cache, v_cache,
+                              phase, phase_id)
+        flash_attention(view(q_pad, n), k_cache, v_cache, view(o_pad, n), tds, phase, W, phase_id, scale=scale)
+        torch.cuda.synchronize()
+        got = o_pad[0, :n].permute(1, 0, 2).cpu().numpy()
+        # the kernel feeds the MFMA with q rounded to the cache's 16-bit type
+        exp = expected_from_stream(q_rot[0][:, lo : lo + n].astype(np.float16), k16, v16, lo + n, n, W, scale)
+        assert_close(got, exp, what=f"positions {lo}..{lo + n - 1}")
+
+    phase.copy_(torch.tensor([PHASE_PREFILL, 0], dtype=torch.uint8))
+    for c in range(2):
+        o, n = ix.prefill_step_integers(c * t, t)
+        offsets.copy_(torch.tensor([o, 0], dtype=torch.int32)), tds.copy_(torch.tensor([n, 0], dtype=torch.int32))
+        step(c * t, t, PHASE_PREFILL)
+    phase.copy_(torch.tensor([PHASE_DECODE, 0], dtype=torch.uint8))
+    o, n = ix.decode_step_integers(2 * t)
+    offsets.copy_(torch.tensor([o, 0], dtype=torch.int32)), tds.copy_(torch.tensor([n, 0], dtype=torch.int32))
+    inp = torch.zeros(1, B, dtype=torch.int32, device=dev)
+    out_tok = torch.zeros(B, 1, dtype=torch.int32, device=dev)
+    for s in range(3):
+        step(2 * t + s, 1, PHASE_DECODE)
+        advance_decode_state(inp, out_tok, offsets, tds, phase)
+    torch.cuda.synchronize()
+    assert offsets.tolist() == [2 * t + 3, 0] and tds.tolist() == [2 * t + 4, 0]

@@ -4,7 +4,7 @@
 
 The reference ships no stored vectors for this path (its compare scripts draw unseeded random
 inputs), so these fixtures are produced by this repository's own fp64 oracle
-(``oracle.attention_ref``), which ``tests/test_oracle_*.py`` pin against closed forms.  Each
+(``oracle.attention_ref``, ``oracle.rope_ref``), which ``tests/test_oracle_*.py`` pin against closed forms.  Each
 ``.npz`` holds the inputs exactly as the kernels see them (fp16 / int) and the fp64 result rounded
 to fp32.  Nothing of the reference is read or executed.
 """
@@ -21,6 +21,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 from oracle import attention_ref as ar  # noqa: E402
 from oracle import index_spec as ix  # noqa: E402
+from oracle import rope_ref as rr  # noqa: E402
 
 CASES = {
     # name: B, H, G, Tq, D, kv_ctx, W, tds, user_phase, launch phase, stage, scale, query_window
@@ -60,11 +61,34 @@ def kv_append_fixture():
     return dict(x=x, cache=cache, cache_offsets=offs, x_rsos=rsos, eps=np.float32(1e-6), expected_plain=plain, expected_rmsnorm=normed)
 
 
+def rope_fixture():
+    """Head dim 256, GQA 8:2, a 5-token chunk per slot at positions up to 30000, ring of 11 rows (wraps), one slot off phase."""
+    rng = np.random.default_rng(23)
+    B, H, G, t, D, T = 3, 8, 2, 5, 256, 11
+    q = rng.standard_normal((B, H, t, D)).astype(np.float32)
+    k = rng.standard_normal((B, G, t, D)).astype(np.float32)
+    v = rng.standard_normal((B, G, t, D)).astype(np.float32)
+    freqs = rr.populate_rope_frequencies_ref(D // 2, 1e6).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    offs = np.array([0, 29998, 8], np.int32)
+    phase = np.array([1, 1, 2], np.uint8)
+    kc = rng.standard_normal((B, G, T, D)).astype(np.float16)
+    vc = rng.standard_normal((B, G, T, D)).astype(np.float16)
+    q_rsos, k_rsos, v_rsos = ((x * x).sum(-1).astype(np.float32) for x in (q, k, v))
+    kc_out, vc_out = kc.copy(), vc.copy()
+    q_rot, k_rot = rr.rope_append_ref(q, k, v, freqs, offs, q_rsos, k_rsos, v_rsos, qw, kw, 1e-6, kc_out, vc_out, phase, 1)
+    return dict(q=q, k=k, v=v, rope_freqs=freqs, cache_offsets=offs, user_phase=phase, q_rsos=q_rsos, k_rsos=k_rsos, v_rsos=v_rsos,
+                q_rmsnorm_w=qw, k_rmsnorm_w=kw, eps=np.float32(1e-6), k_cache=kc, v_cache=vc, phase=np.int32(1),
+                expected_q=q_rot, expected_k=k_rot, expected_k_cache=kc_out, expected_v_cache=vc_out)
+
+
 def main():
     for name in CASES:
         np.savez_compressed(os.path.join(HERE, f"attn_{name}.npz"), **build(name))
     np.savez_compressed(os.path.join(HERE, "kv_append_ref_case.npz"), **kv_append_fixture())
-    print("wrote", len(CASES) + 1, "fixtures to", HERE)
+    np.savez_compressed(os.path.join(HERE, "rope_append_case.npz"), **rope_fixture())
+    print("wrote", len(CASES) + 2, "fixtures to", HERE)
 
 
 if __name__ == "__main__":

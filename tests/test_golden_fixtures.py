@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from oracle import attention_ref as ar
+from oracle import rope_ref as rr
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 ATTN = sorted(glob.glob(os.path.join(GOLDEN, "attn_*.npz")))
@@ -14,6 +15,7 @@ ATTN = sorted(glob.glob(os.path.join(GOLDEN, "attn_*.npz")))
 
 def test_fixtures_present():
     assert len(ATTN) >= 5 and os.path.exists(os.path.join(GOLDEN, "kv_append_ref_case.npz"))
+    assert os.path.exists(os.path.join(GOLDEN, "rope_append_case.npz"))
 
 
 @pytest.mark.parametrize("path", ATTN, ids=[os.path.basename(p)[5:-4] for p in ATTN])
@@ -81,3 +83,38 @@ def test_kv_append_matches_fixture(gpu_device):
     got, exp = cache.cpu().numpy().astype(np.float32), f["expected_rmsnorm"].astype(np.float32)
     np.testing.assert_allclose(got, exp, rtol=1e-3, atol=1e-6)
     assert np.array_equal(got == f["cache"].astype(np.float32), exp == f["cache"].astype(np.float32))
+
+
+def _rope_fixture():
+    return np.load(os.path.join(GOLDEN, "rope_append_case.npz"))
+
+
+def test_oracle_reproduces_rope_fixture():
+    f = _rope_fixture()
+    kc, vc = f["k_cache"].copy(), f["v_cache"].copy()
+    q_rot, k_rot = rr.rope_append_ref(f["q"], f["k"], f["v"], f["rope_freqs"], f["cache_offsets"], f["q_rsos"], f["k_rsos"], f["v_rsos"],
+                                      f["q_rmsnorm_w"], f["k_rmsnorm_w"], float(f["eps"]), kc, vc, f["user_phase"], int(f["phase"]))
+    assert np.array_equal(q_rot, f["expected_q"]) and np.array_equal(k_rot, f["expected_k"])
+    assert np.array_equal(kc, f["expected_k_cache"]) and np.array_equal(vc, f["expected_v_cache"])
+
+
+@pytest.mark.gpu
+def test_rope_kernels_match_fixture(gpu_device):
+    import torch
+
+    from g4b_amd.kernels.rope import apply_rope, apply_rope_and_append
+
+    f = _rope_fixture()
+    t = lambda name: torch.from_numpy(f[name]).to(gpu_device)
+    q, k = t("q"), t("k")
+    apply_rope(q, k, t("rope_freqs"), t("cache_offsets"), t("q_rsos"), t("k_rsos"), t("q_rmsnorm_w"), t("k_rmsnorm_w"), float(f["eps"]))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(q.cpu().numpy(), f["expected_q"], rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(k.cpu().numpy(), f["expected_k"], rtol=2e-5, atol=2e-5)
+    q, k, kc, vc = t("q"), t("k"), t("k_cache"), t("v_cache")
+    apply_rope_and_append(q, k, t("v"), t("rope_freqs"), t("cache_offsets"), t("q_rsos"), t("k_rsos"), t("v_rsos"), t("q_rmsnorm_w"),
+                          t("k_rmsnorm_w"), float(f["eps"]), kc, vc, t("user_phase"), int(f["phase"]))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(kc.float().cpu().numpy(), f["expected_k_cache"].astype(np.float32), rtol=2e-3, atol=2e-3)
+    np.testing.assert_allclose(vc.float().cpu().numpy(), f["expected_v_cache"].astype(np.float32), rtol=2e-3, atol=2e-3)
+    assert np.array_equal(kc[2].cpu().numpy(), f["k_cache"][2])  # off-phase slot

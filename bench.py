@@ -85,7 +85,8 @@ class BatchedDecode(Workload):
 
     bound = "hbm"
 
-    def __init__(self, device, B=64, kv_ctx=32768, len_lo=128, len_hi=32768, swa_every=2, seed=0, name="decode_batched_b64"):
+    def __init__(self, device, B=64, kv_ctx=32768, len_lo=128, len_hi=32768, swa_every=2, seed=0, name="decode_batched_b64",
+                 heads=H, groups=G, dim=D):
         import numpy as np
         import torch
 
@@ -94,22 +95,24 @@ class BatchedDecode(Workload):
         self.name = name
         self.fa2 = fa2
         self.B, self.kv_ctx = B, kv_ctx
+        H_, G_, D_ = heads, groups, dim
+        self.G_, self.D_ = G_, D_
         rng = np.random.default_rng(seed)
         self.tds_list = rng.integers(len_lo, len_hi + 1, B).tolist()
         self.win_list = [512 if (swa_every and b % swa_every == 0) else kv_ctx for b in range(B)]
         self.n_keys = [min(t, w) for t, w in zip(self.tds_list, self.win_list)]
-        self.q = _randn_f16((B, H, 1, D), seed + 1, device)
-        self.k = _randn_f16((B, G, kv_ctx, D), seed + 2, device)
-        self.v = _randn_f16((B, G, kv_ctx, D), seed + 3, device)
+        self.q = _randn_f16((B, H_, 1, D_), seed + 1, device)
+        self.k = _randn_f16((B, G_, kv_ctx, D_), seed + 2, device)
+        self.v = _randn_f16((B, G_, kv_ctx, D_), seed + 3, device)
         self.o = torch.empty_like(self.q)
         self.tds = torch.tensor(self.tds_list, dtype=torch.int32, device=device)
         self.win = torch.tensor(self.win_list, dtype=torch.int32, device=device)
         self.phase = torch.full((B,), fa2.PHASE_DECODE, dtype=torch.uint8, device=device)
-        self.ws = torch.empty(fa2.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device=device)
+        self.ws = torch.empty(fa2.workspace_bytes(B, H_, G_, 1, D_), dtype=torch.uint8, device=device)
         self.plans = {}  # bound calls (arguments validated once), one per kernel_mask
         # algorithmic bytes: every visible K and V row once per kv head (2 * G * D * 2 bytes per key)
-        self.bytes = 2 * G * D * 2 * sum(self.n_keys)
-        self.flops = 4 * H * D * sum(self.n_keys)
+        self.bytes = 2 * G_ * D_ * 2 * sum(self.n_keys)
+        self.flops = 4 * H_ * D_ * sum(self.n_keys)
         self.units = self.bytes
 
     def launch(self, i=0, kernel_mask=0):
@@ -133,7 +136,7 @@ class BatchedDecode(Workload):
         t0 = time.perf_counter()
         ar.attention_cpu_baseline(q, k, v, tds, [2] * len(slots), self.kv_ctx, 2, scale=SCALE, window_sizes=win)
         dt = time.perf_counter() - t0
-        done = 2 * G * D * 2 * sum(self.n_keys[b] for b in slots)
+        done = 2 * self.G_ * self.D_ * 2 * sum(self.n_keys[b] for b in slots)
         return dt, done, f"slots 0..{len(slots) - 1} of {self.B} ({done / 1e6:.1f} MB of KV), one pass"
 
 
@@ -348,6 +351,8 @@ class RopeAppend(Workload):
 
 WORKLOADS = {
     "decode_batched": lambda dev: BatchedDecode(dev),
+    # head dimension 512 (global-attention layers): 32 sequences, every slot attends its whole history
+    "decode_batched_d512": lambda dev: BatchedDecode(dev, B=32, swa_every=0, dim=512, name="decode_batched_b32_d512"),
     "decode_single": lambda dev: SingleDecode(dev),
     "prefill_causal_2048": lambda dev: Prefill(dev, 2048),
     "prefill_causal_8192": lambda dev: Prefill(dev, 8192),
@@ -483,6 +488,7 @@ def main():
             torch.cuda.empty_cache()
 
     primary_is_hbm = res["roofline"]["bound"] == "hbm"
+    head_dim = 512 if args.workload.endswith("_d512") else D
     line = {
         "metric": METRIC,
         "value": round(res["GBps"] if primary_is_hbm else res["TFLOPs"], 2),
@@ -496,7 +502,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": args.workload, "H": H, "G": G, "D": D, "scale": SCALE,
+        "config": {"workload": args.workload, "H": H, "G": G, "D": head_dim, "scale": SCALE,
                    "detail": "fp16 Q/K/V ~ N(0,1) seeded, fp32 softmax accumulation"},
         "roofline": res["roofline"],
         "cpu_baseline": cpu,

@@ -21,6 +21,8 @@ int fail(int code, const char* fmt, ...) {
 }
 
 constexpr int kDefaultWorkers = 1024;  // 256 CUs x 4 SIMDs x 1 wave
+// a worker for head dimension 512 is a workgroup of two waves
+int default_workers(int D) { return D > 256 ? kDefaultWorkers * 256 / D : kDefaultWorkers; }
 constexpr int kMaxDecodeRows = 16;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -57,7 +59,7 @@ uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, i
     if (B < 1 || H < 1 || G < 1 || Tq < 1 || D < 1 || H % G) return 0;
     const int64_t rows = (int64_t)(H / G) * Tq;
     if (rows > kMaxDecodeRows) return prefill_workspace_bytes(H, G, Tq, D);
-    const int nw = num_workers > 0 ? num_workers : kDefaultWorkers;
+    const int nw = num_workers > 0 ? num_workers : default_workers(D);
     return decode_slots(B, G, nw) * (uint64_t)rows * (uint64_t)(D + 2) * sizeof(float);
 }
 
@@ -72,7 +74,8 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     if (a->B < 1 || a->H < 1 || a->G < 1 || a->Tq < 1 || a->D < 1 || a->KV_CTX < 1)
         return fail(G4B_ERR_INVALID_ARGUMENT, "B, H, G, Tq, D, KV_CTX must be positive");
     if (a->H % a->G) return fail(G4B_ERR_INVALID_ARGUMENT, "H (%d) must be a multiple of G (%d)", a->H, a->G);
-    if (a->D != 128 && a->D != 256) return fail(G4B_ERR_UNSUPPORTED, "head_dim %d not built (128 and 256 are)", a->D);
+    if (a->D != 128 && a->D != 256 && a->D != 512)
+        return fail(G4B_ERR_UNSUPPORTED, "head_dim %d not built (128, 256 and 512 are)", a->D);
     if (a->B > 65535 || a->G > 65535) return fail(G4B_ERR_UNSUPPORTED, "B and G must be <= 65535");
     if (a->ctx_window_size < 1 || a->ctx_window_size > a->KV_CTX)
         return fail(G4B_ERR_INVALID_ARGUMENT, "ctx_window_size (%d) must be in [1, KV_CTX = %d]", a->ctx_window_size, a->KV_CTX);
@@ -133,7 +136,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     hipError_t e;
     if (rows <= kMaxDecodeRows) {
         if (a->workspace) {
-            const int nw = a->num_workers > 0 ? a->num_workers : kDefaultWorkers;
+            const int nw = a->num_workers > 0 ? a->num_workers : default_workers(a->D);
             const uint64_t need = g4b_attn_workspace_bytes(a->B, a->H, a->G, a->Tq, a->D, nw);
             if (a->workspace_bytes < need)
                 return fail(G4B_ERR_WORKSPACE, "workspace holds %llu bytes, %llu needed for %d workers",
@@ -148,6 +151,8 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
         if (128 % p.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide 128 for prefill-shaped launches", p.R);
+        if (a->D == 512)
+            return fail(G4B_ERR_UNSUPPORTED, "head_dim 512 is built for launches of at most %d query rows per kv head", kMaxDecodeRows);
         p.split_slots = 0;
         const uint64_t need = prefill_workspace_bytes(a->H, a->G, a->Tq, a->D);
         if (a->workspace && need) {

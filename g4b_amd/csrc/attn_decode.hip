@@ -44,17 +44,23 @@ G4B_DEV float pick(const f4& c, int e, int cls) {
 
 // One segment: tiles [t0, t1) of pair (bb, g) whose slot has tlb tiles per kv head.  Worker w
 // writes the output itself when the segment is the whole pair, else partial slot (w + pair).
-template <int D, int CL, class T>
-G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb) {
+//
+// DH > 1: the workgroup has DH waves and wave hv owns columns [hv*D/DH, (hv+1)*D/DH) of the head dimension: its share
+// of q, of every K and V row and of the output.  The waves add their partial dot products through LDS once per tile
+// and then run the same softmax, so the register tiling is that of head dimension D/DH.
+template <int D, int CL, class T, int DH>
+G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb, float* xch) {
+    constexpr int DL = D / DH;         // columns this wave owns
     constexpr int E = 4 / CL;          // scores a lane keeps per 16-row MFMA tile
     constexpr int KT = 16 / CL;        // keys per MFMA tile
     constexpr int NT = DEC_TILE / KT;  // MFMA tiles per 32 keys
-    constexpr int PIECES = D / 8;      // 16-byte pieces per key row
+    constexpr int PIECES = DL / 8;     // 16-byte pieces of a key row this wave reads
     constexpr int NC = PIECES / (4 * CL);
-    constexpr int DC = D / 128;
+    constexpr int DC = DL / 128;
     constexpr int ROWB = D * 2;  // bytes per cache row
     static_assert(NC >= 1 && DC >= 1, "head dim too small for this tiling");
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int hv = (DH > 1) ? (int)(threadIdx.x >> 6) : 0;
     const int m16 = lane & 15, g4 = lane >> 4;
     const int cls = m16 % CL;
     const int G = p.G, Tq = p.Tq;
@@ -63,9 +69,9 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
     const SlotInfo si = slot_info(p, bb);
     const int KV_CTX = p.KV_CTX;
     const char* kbase =
-        static_cast<const char*>(p.k) + ((int64_t)bb * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
+        static_cast<const char*>(p.k) + ((int64_t)bb * p.k_sb + (int64_t)g * KV_CTX * D + hv * DL) * 2;
     const char* vbase =
-        static_cast<const char*>(p.v) + ((int64_t)bb * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
+        static_cast<const char*>(p.v) + ((int64_t)bb * p.v_sb + (int64_t)g * KV_CTX * D + hv * DL) * 2;
 
     // this lane's query row (as MFMA column n = m16 = row*CL + cls)
     const int row = m16 / CL;
@@ -80,7 +86,8 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
 
     u4 qf[NC];
     {
-        const int64_t qoff = (int64_t)bb * p.q_s[0] + (int64_t)(g * p.R + hh) * p.q_s[1] + (int64_t)ti * p.q_s[2];
+        const int64_t qoff =
+            (int64_t)bb * p.q_s[0] + (int64_t)(g * p.R + hh) * p.q_s[1] + (int64_t)ti * p.q_s[2] + hv * DL;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int piece = cls + CL * g4 + 4 * CL * c;
@@ -125,6 +132,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
 
     load_k(t0);
     load_v(t0);
+    if constexpr (DH > 1) __syncthreads();  // the exchange buffers of the previous segment are free
     for (int t = t0; t < t1; ++t) {
         const int jb = si.klo + t * DEC_TILE;
         // ---- S^T = K Q^T -------------------------------------------------------
@@ -143,6 +151,20 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
             }
         }
         if (t + 1 < t1) load_k(t + 1);
+        if constexpr (DH > 1) {
+            // add the other waves' partial dot products; buffers alternate so one barrier per tile is enough
+            float* xb = xch + (t & 1) * (DH * 8 * 64);
+#pragma unroll
+            for (int s = 0; s < 8; ++s) xb[(hv * 8 + s) * 64 + lane] = sc[s];
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                float x = 0.f;
+#pragma unroll
+                for (int h = 0; h < DH; ++h) x += xb[(h * 8 + s) * 64 + lane];  // same order in every wave
+                sc[s] = x;
+            }
+        }
 
         // ---- online softmax (per row; a row's keys are spread over the 4 lane groups)
         if (jb < lo_max || jb + DEC_TILE > hi_min) {
@@ -199,7 +221,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
                     float v8[8];
 #pragma unroll
                     for (int jj = 0; jj < 8; ++jj) v8[jj] = pick<CL>(acc[dc * 8 + jj], e, cls) * inv;
-                    const int d0 = 128 * dc + (4 * g4 + e * CL + cls) * 8;
+                    const int d0 = hv * DL + 128 * dc + (4 * g4 + e * CL + cls) * 8;
                     store8(p.o, ooff + d0, p.o_dt, v8);
                 }
             }
@@ -213,11 +235,11 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
                     float v8[8];
 #pragma unroll
                     for (int jj = 0; jj < 8; ++jj) v8[jj] = pick<CL>(acc[dc * 8 + jj], e, cls);
-                    const int d0 = 128 * dc + (4 * g4 + e * CL + cls) * 8;
+                    const int d0 = hv * DL + 128 * dc + (4 * g4 + e * CL + cls) * 8;
                     store8(po, d0, DT_F32, v8);
                 }
             }
-            if (cls == 0 && g4 == 0) {
+            if (cls == 0 && g4 == 0 && hv == 0) {
                 float* pm = p.part_ml + (slot * NR + row) * 2;
                 pm[0] = m_run;
                 pm[1] = l_tot;
@@ -226,9 +248,11 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
     }
 }
 
-template <int D, int CL, class T>
-__global__ __launch_bounds__(64, 1) void attn_decode_worker(const AttnParams p) {
-    const int lane = threadIdx.x;
+template <int D, int CL, class T, int DH>
+__global__ __launch_bounds__(64 * DH, 1) void attn_decode_worker(const AttnParams p) {
+    __shared__ float xch_buf[DH > 1 ? 2 * DH * 8 * 64 : 1];
+    float* xch = xch_buf;
+    const int lane = threadIdx.x & 63;  // every wave of the workgroup does the same bookkeeping
     const int w = blockIdx.x;
     const int B = p.B, G = p.G;
 
@@ -236,7 +260,7 @@ __global__ __launch_bounds__(64, 1) void attn_decode_worker(const AttnParams p) 
         // no workspace: worker w owns the whole pair w
         const int bb = w / G, g = w % G;
         const int tlb = slot_tiles(p, bb);
-        if (tlb > 0) decode_segment<D, CL, T>(p, w, bb, g, 0, tlb, tlb);
+        if (tlb > 0) decode_segment<D, CL, T, DH>(p, w, bb, g, 0, tlb, tlb, xch);
         return;
     }
 
@@ -271,7 +295,7 @@ __global__ __launch_bounds__(64, 1) void attn_decode_worker(const AttnParams p) 
                 const int64_t fs = (int64_t)ex + (int64_t)g * tlb;
                 const int t0 = (int)(max(ws, fs) - fs);
                 const int t1 = (int)(min(we, fs + tlb) - fs);
-                if (t1 > t0) decode_segment<D, CL, T>(p, w, bb, g, t0, t1, tlb);
+                if (t1 > t0) decode_segment<D, CL, T, DH>(p, w, bb, g, t0, t1, tlb, xch);
             }
         }
         carry += __shfl(incl, 63);
@@ -334,36 +358,45 @@ __global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
     const float msafe = (mref == -INFINITY) ? 0.f : mref;
 
     // pass 2: wave k takes workers w0 + k, w0 + k + 4, ...; a lane owns four output columns
-    constexpr int LPR = D / 4;  // lanes that hold a row
+    constexpr int LPR = D / 4 < 64 ? D / 4 : 64;  // lanes that hold a row
+    constexpr int NV = D / 4 / LPR;               // float4 pieces per lane: piece v covers columns (v*64 + lane)*4..+3
     constexpr int UN = 8;
-    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    f4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = f4{0.f, 0.f, 0.f, 0.f};
     float l = 0.f;
     for (int wb = w0 + wave; wb <= w1; wb += 4 * UN) {
         float wgt[UN], lw[UN];
-        f4 ov[UN];
+        f4 ov[UN][NV];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int w = min(wb + 4 * u, w1);  // clamped loads, masked below
             const float* ml = ml_of(w);
             wgt[u] = ml[0];
             lw[u] = ml[1];
-            ov[u] = (lane < LPR) ? *reinterpret_cast<const f4*>(p.part_o + (((int64_t)w + pair) * NR + row) * D + lane * 4)
-                                 : f4{0.f, 0.f, 0.f, 0.f};
+            const float* po = p.part_o + (((int64_t)w + pair) * NR + row) * D;
+#pragma unroll
+            for (int v = 0; v < NV; ++v)
+                ov[u][v] = (lane < LPR) ? *reinterpret_cast<const f4*>(po + (v * 64 + lane) * 4) : f4{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const bool live = (wb + 4 * u <= w1) && (wgt[u] != -INFINITY);
             const float e = live ? fast_exp2(wgt[u] - msafe) : 0.f;
             if (live) {
-                acc += ov[u] * e;
+#pragma unroll
+                for (int v = 0; v < NV; ++v) acc[v] += ov[u][v] * e;
                 l += lw[u] * e;
             }
         }
     }
-    if (lane < LPR) sm_acc[wave][lane] = acc;
+    if (lane < LPR) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) sm_acc[wave][v * 64 + lane] = acc[v];
+    }
     if (lane == 0) sm_l[wave] = l;
     __syncthreads();
-    if (tid < LPR) {
+    if (tid < D / 4) {
         const f4 r = sm_acc[0][tid] + sm_acc[1][tid] + sm_acc[2][tid] + sm_acc[3][tid];
         const float lt = sm_l[0] + sm_l[1] + sm_l[2] + sm_l[3];
         const float inv = lt > 0.f ? 1.f / lt : 0.f;
@@ -373,8 +406,10 @@ __global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
 
 template <int D, int CL, class T>
 static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
+    constexpr int DH = D > 256 ? D / 256 : 1;  // waves per worker: each owns at most 256 columns
     if (p.kernel_mask & 1) {
-        hipLaunchKernelGGL((attn_decode_worker<D, CL, T>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((attn_decode_worker<D, CL, T, DH>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64 * DH), 0, stream,
+                           p);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -392,9 +427,11 @@ static hipError_t launch_decode_cl(const AttnParams& p, hipStream_t stream) {
 
 hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream) {
     if (kv_dt == DT_F16) {
+        if (D == 512) return launch_decode_cl<512, F16>(p, stream);
         if (D == 256) return launch_decode_cl<256, F16>(p, stream);
         if (D == 128) return launch_decode_cl<128, F16>(p, stream);
     } else {
+        if (D == 512) return launch_decode_cl<512, BF16>(p, stream);
         if (D == 256) return launch_decode_cl<256, BF16>(p, stream);
         if (D == 128) return launch_decode_cl<128, BF16>(p, stream);
     }

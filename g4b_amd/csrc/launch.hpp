@@ -7,9 +7,9 @@
 
 namespace g4b {
 
-// rows = (H/G) * Tq <= 16, D in {128, 256}; kv_dt in {DT_F16, DT_BF16}
+// rows = (H/G) * Tq <= 16, D in {128, 256, 512}; kv_dt in {DT_F16, DT_BF16}
 hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
-// any Tq; (H/G) must divide 128
+// any Tq; (H/G) must divide 128; D in {128, 256}
 hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
 
 struct KvAppendParams {

@@ -28,7 +28,7 @@ extern "C" {
 enum g4b_status {
     G4B_OK = 0,
     G4B_ERR_INVALID_ARGUMENT = -1, /* shape / stride / dtype / value check failed (reference: tl.static_assert) */
-    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim 512, STAGE_ON_BAND alone) */
+    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim 512 with more than 16 query rows per kv head, STAGE_ON_BAND alone) */
     G4B_ERR_WORKSPACE = -3,        /* workspace missing or too small for the requested split-KV launch */
     G4B_ERR_LAUNCH = -4            /* the HIP runtime refused the launch (no device, bad stream, ...) */
 };

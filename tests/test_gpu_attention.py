@@ -32,6 +32,9 @@ DECODE_CASES = [
     ("decode_biggroup_w4096", 4, 32, 4, 256, 4096),
     ("decode_mha_w512", 3, 4, 4, 128, 512),
     ("decode_group16_w2048", 2, 16, 1, 256, 2048),
+    ("decode_d512_w2048", 4, 16, 4, 512, 2048),
+    ("decode_d512_group8_w1024", 2, 16, 2, 512, 1024),
+    ("decode_d512_group16_w700", 3, 16, 1, 512, 700),
 ]
 
 
@@ -85,6 +88,22 @@ def test_small_query_blocks_take_the_streaming_kernel(fa, Tq, H, G):
             fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, *parts, stage=stage, scale=0.0625)
             torch.cuda.synchronize()
             assert_close(o.float().cpu().numpy(), ref, what=f"Tq={Tq} stage={stage} split={bool(parts)}")
+
+
+@pytest.mark.parametrize("Tq,H,G", [(2, 8, 2), (4, 8, 2), (3, 4, 4), (1, 16, 1)])
+@pytest.mark.parametrize("num_workers", [0, 5, 2048])
+def test_head_dim_512_query_blocks_and_worker_counts(fa, Tq, H, G, num_workers):
+    """Head dimension 512 (the global-attention layers): two waves per worker share the dot product."""
+    B, D, kv_ctx, W = 3, 512, 300, 260
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=31)
+    tds = [Tq, 260, 260 + 91]
+    phase = [1] * B
+    ref = oracle(q, k, v, tds, phase, W, 1, scale=0.0442)
+    ws = torch.empty(fa.workspace_bytes(B, H, G, Tq, D, num_workers), dtype=torch.uint8, device="cuda")
+    o.fill_(777.0)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, scale=0.0442, workspace=ws, num_workers=num_workers)
+    torch.cuda.synchronize()
+    assert_close(o.float().cpu().numpy(), ref, what=f"D=512 Tq={Tq} workers={num_workers}")
 
 
 PREFILL_CASES = [

@@ -192,7 +192,7 @@ class Prefill(Workload):
 
     bound = "mfma"
 
-    def __init__(self, device, S, query_window=None, seed=0):
+    def __init__(self, device, S, query_window=None, seed=0, dim=D):
         import torch
 
         from g4b_amd.kernels import fa2
@@ -200,9 +200,12 @@ class Prefill(Workload):
         self.fa2 = fa2
         self.S, self.qw = S, query_window
         self.name = f"prefill_causal_{S}" if query_window is None else f"prefill_swa{query_window}_{S}"
-        self.q = _randn_f16((1, H, S, D), seed + 1, device)
-        self.k = _randn_f16((1, G, S, D), seed + 2, device)
-        self.v = _randn_f16((1, G, S, D), seed + 3, device)
+        D_ = self.D_ = dim
+        if dim != D:
+            self.name += f"_d{dim}"
+        self.q = _randn_f16((1, H, S, D_), seed + 1, device)
+        self.k = _randn_f16((1, G, S, D_), seed + 2, device)
+        self.v = _randn_f16((1, G, S, D_), seed + 3, device)
         self.o = torch.empty_like(self.q)
         self.tds = torch.full((1,), S, dtype=torch.int32, device=device)
         self.phase = torch.full((1,), fa2.PHASE_PREFILL, dtype=torch.uint8, device=device)
@@ -213,8 +216,8 @@ class Prefill(Workload):
             pairs = w * (w + 1) // 2 + (S - w) * w
         self.pairs = pairs
         self.plan = None
-        self.flops = 4 * H * D * pairs
-        self.bytes = (2 * H * S * D + 2 * G * S * D) * 2
+        self.flops = 4 * H * D_ * pairs
+        self.bytes = (2 * H * S * D_ + 2 * G * S * D_) * 2
         self.units = self.flops
 
     def launch(self, i=0, kernel_mask=0):
@@ -240,7 +243,7 @@ class Prefill(Workload):
         else:
             pairs = sum(min(self.qw, self.S - rows + i + 1) for i in range(rows))
         # the dense CPU formulation computes every (row, key) score, masked or not
-        return dt, 4 * H * D * pairs, f"last {rows} query rows against all {self.S} keys (dense scores)"
+        return dt, 4 * H * self.D_ * pairs, f"last {rows} query rows against all {self.S} keys (dense scores)"
 
 
 class MixedStep(Workload):
@@ -357,6 +360,7 @@ WORKLOADS = {
     "prefill_causal_2048": lambda dev: Prefill(dev, 2048),
     "prefill_causal_8192": lambda dev: Prefill(dev, 8192),
     "prefill_swa_8192": lambda dev: Prefill(dev, 8192, query_window=512),
+    "prefill_causal_8192_d512": lambda dev: Prefill(dev, 8192, dim=512),
     "mixed_step": lambda dev: MixedStep(dev),
     "rope_append": lambda dev: RopeAppend(dev),
 }

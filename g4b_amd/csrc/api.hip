@@ -34,17 +34,18 @@ uint64_t decode_slots(int B, int G, int nw) { return (uint64_t)nw + (uint64_t)B 
 // slots bring fewer workgroups than the chip has CUs splits the keys of every item; 0 = the shape never splits.
 constexpr int kPrefillFillWorkgroups = 256;
 constexpr int kPrefillMaxSplitSlots = 64;
-int prefill_split_slots(int H, int G, int Tq) {
-    const int R = H / G;
-    if (R < 1 || 128 % R) return 0;
-    const int tokb = 128 / R;
+int prefill_rows_per_workgroup(int D) { return D > 256 ? 64 : 128; }
+int prefill_split_slots(int H, int G, int Tq, int D) {
+    const int R = H / G, bm = prefill_rows_per_workgroup(D);
+    if (R < 1 || bm % R) return 0;
+    const int tokb = bm / R;
     const int64_t per_slot = (int64_t)((Tq + tokb - 1) / tokb) * G;  // workgroups one slot brings
     const int64_t slots = kPrefillFillWorkgroups / per_slot;
     if (slots < 2) return 0;
     return (int)(slots < kPrefillMaxSplitSlots ? slots : kPrefillMaxSplitSlots);
 }
 uint64_t prefill_workspace_bytes(int H, int G, int Tq, int D) {
-    return (uint64_t)prefill_split_slots(H, G, Tq) * (uint64_t)H * (uint64_t)Tq * (uint64_t)(D + 2) * sizeof(float);
+    return (uint64_t)prefill_split_slots(H, G, Tq, D) * (uint64_t)H * (uint64_t)Tq * (uint64_t)(D + 2) * sizeof(float);
 }
 
 }  // namespace
@@ -150,9 +151,9 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         }
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
-        if (128 % p.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide 128 for prefill-shaped launches", p.R);
-        if (a->D == 512)
-            return fail(G4B_ERR_UNSUPPORTED, "head_dim 512 is built for launches of at most %d query rows per kv head", kMaxDecodeRows);
+        const int bm = prefill_rows_per_workgroup(a->D);
+        if (bm % p.R)
+            return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide %d for prefill-shaped launches with head_dim %d", p.R, bm, a->D);
         p.split_slots = 0;
         const uint64_t need = prefill_workspace_bytes(a->H, a->G, a->Tq, a->D);
         if (a->workspace && need) {
@@ -160,11 +161,12 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
                 return fail(G4B_ERR_WORKSPACE, "workspace holds %llu bytes, %llu needed to split this prefill shape",
                             (unsigned long long)a->workspace_bytes, (unsigned long long)need);
             if (!aligned16(a->workspace)) return fail(G4B_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
-            p.split_slots = prefill_split_slots(a->H, a->G, a->Tq);
+            p.split_slots = prefill_split_slots(a->H, a->G, a->Tq, a->D);
             p.part_o = static_cast<float*>(a->workspace);
             p.part_ml = p.part_o + (uint64_t)p.split_slots * a->H * a->Tq * a->D;
         }
-        e = g4b::launch_attn_prefill(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
+        e = a->D == 512 ? g4b::launch_attn_prefill_wide(p, a->kv_dtype, static_cast<hipStream_t>(stream))
+                        : g4b::launch_attn_prefill(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     }
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
     return G4B_OK;

@@ -27,6 +27,7 @@
 // rescaled lazily.
 #include "common.hpp"
 #include "launch.hpp"
+#include "prefill_combine.hpp"
 #include "prefill_map.hpp"
 
 namespace g4b {
@@ -460,61 +461,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
             }
         }
     }
-}
-
-// Merge the key splits of a prefill-shaped launch: a lane per four output columns of a row, PFC_ROWS rows per
-// workgroup, every load of a row independent of the others.
-constexpr int PFC_ROWS = 8;
-template <int D, int NS>
-G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, int tb, int nsplit) {
-    constexpr int LPR = D / 4;      // lanes per row
-    constexpr int RPP = 256 / LPR;  // rows per pass
-    const int r_in = threadIdx.x / LPR, d0 = (threadIdx.x % LPR) * 4;
-#pragma unroll
-    for (int pass = 0; pass < PFC_ROWS / RPP; ++pass) {
-        const int t = tb * PFC_ROWS + pass * RPP + r_in;
-        if (t >= p.Tq) continue;
-        float ms[NS], ls[NS];
-        f4 ov[NS];
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            const int64_t prow = ((int64_t)(a_idx * nsplit + min(s, nsplit - 1)) * p.H + h) * p.Tq + t;  // clamped, masked below
-            ms[s] = p.part_ml[prow * 2];
-            ls[s] = (s < nsplit) ? p.part_ml[prow * 2 + 1] : 0.f;
-            ov[s] = *reinterpret_cast<const f4*>(p.part_o + prow * D + d0);
-        }
-        float mref = -INFINITY;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-            if (ls[s] > 0.f) mref = fmaxf(mref, ms[s]);
-        f4 acc = {0.f, 0.f, 0.f, 0.f};
-        float l = 0.f;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-            if (ls[s] > 0.f) {
-                const float w = fast_exp2(ms[s] - mref);
-                acc += ov[s] * w;
-                l += ls[s] * w;
-            }
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)h * p.o_s[1] + (int64_t)t * p.o_s[2] + d0;
-        store4(p.o, ooff, p.o_dt, acc * inv);
-    }
-}
-
-template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
-    __shared__ int sh_scan[8];
-    const int tblocks = (p.Tq + PFC_ROWS - 1) / PFC_ROWS;
-    const int a_idx = blockIdx.x / (p.H * tblocks), h = (blockIdx.x / tblocks) % p.H, tb = blockIdx.x % tblocks;
-    int n_active;
-    const int b = nth_active_slot(p, a_idx, n_active, sh_scan);
-    const int nsplit = prefill_splits(p.split_slots, n_active);
-    if (b < 0 || nsplit == 1) return;
-    if (nsplit <= 2) prefill_combine_rows<D, 2>(p, a_idx, b, h, tb, nsplit);
-    else if (nsplit <= 4) prefill_combine_rows<D, 4>(p, a_idx, b, h, tb, nsplit);
-    else if (nsplit <= 8) prefill_combine_rows<D, 8>(p, a_idx, b, h, tb, nsplit);
-    else prefill_combine_rows<D, 16>(p, a_idx, b, h, tb, nsplit);
 }
 
 template <int D, class T>

@@ -45,8 +45,8 @@ __host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int&
 
 // Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on
 // the device and surplus workgroups leave at once.
-inline int prefill_grid(const AttnParams& p) {
-    const int tokb = PF_BM / p.R;
+inline int prefill_grid(const AttnParams& p, int bm = PF_BM) {
+    const int tokb = bm / p.R;
     const int nq = (p.Tq + tokb - 1) / tokb;
     const int slots = p.part_o ? p.split_slots : 1;
     int blocks = 0;

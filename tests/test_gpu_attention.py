@@ -115,7 +115,14 @@ PREFILL_CASES = [
     ("prefill_ragged_t100", 2, 8, 2, 100, 600, 256, 512, ix.STAGE_CAUSAL),
     ("prefill_mha_t70", 1, 2, 2, 70, 300, 128, 300, ix.STAGE_CAUSAL),
     ("prefill_group8_t48", 1, 16, 2, 48, 500, 256, 400, ix.STAGE_CAUSAL),
+    # head dimension 512: a pair of waves shares each 32-row block
+    ("prefill_d512_t128_w1024", 2, 8, 2, 128, 1024, 512, 1024, ix.STAGE_CAUSAL),
+    ("prefill_d512_ragged_t100", 2, 8, 2, 100, 600, 512, 512, ix.STAGE_CAUSAL),
+    ("full_d512_t96_w256", 2, 16, 4, 96, 256, 512, 256, ix.STAGE_FULL),
+    ("prefill_d512_group8_t48", 1, 16, 2, 48, 500, 512, 400, ix.STAGE_CAUSAL),
+    ("prefill_d512_mha_t70", 1, 2, 2, 70, 300, 512, 300, ix.STAGE_CAUSAL),
 ]
+SPLIT_CASES = PREFILL_CASES[:3] + PREFILL_CASES[4:5] + PREFILL_CASES[7:9]
 
 
 @pytest.mark.parametrize("case", PREFILL_CASES, ids=[c[0] for c in PREFILL_CASES])
@@ -132,7 +139,7 @@ def test_prefill_matches_oracle(fa, case, scale):
     assert_close(o.float().cpu().numpy(), ref, what=name)
 
 
-@pytest.mark.parametrize("case", PREFILL_CASES[:3] + PREFILL_CASES[4:5], ids=[c[0] for c in PREFILL_CASES[:3] + PREFILL_CASES[4:5]])
+@pytest.mark.parametrize("case", SPLIT_CASES, ids=[c[0] for c in SPLIT_CASES])
 def test_prefill_key_split_agrees_with_one_workgroup_per_tile(fa, case):
     """Shapes that bring few workgroups split every item's keys over several and merge the partials; with
     ``workspace=False`` nothing is split.  Both must match the oracle and each other."""

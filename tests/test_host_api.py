@@ -115,9 +115,9 @@ def test_python_boundary_validates_like_the_reference(native):
     q5, k5 = torch.zeros(2, 8, 1, 192, dtype=torch.float16), torch.zeros(2, 2, 64, 192, dtype=torch.float16)
     with pytest.raises(NotImplementedError, match="head_dim"):
         flash_attention(q5, k5, k5, q5.clone(), tds, ph, 64, PHASE_DECODE)
-    # head dimension 512 is built for the streaming kernel only (at most 16 query rows per kv head)
-    q6, k6 = torch.zeros(2, 8, 8, 512, dtype=torch.float16), torch.zeros(2, 2, 64, 512, dtype=torch.float16)
-    with pytest.raises(NotImplementedError, match="head_dim 512"):
+    # prefill-shaped launches: the group size must divide the rows of a workgroup (64 for head dimension 512)
+    q6, k6 = torch.zeros(2, 6, 8, 512, dtype=torch.float16), torch.zeros(2, 2, 64, 512, dtype=torch.float16)
+    with pytest.raises(NotImplementedError, match="must divide 64"):
         flash_attention(q6, k6, k6, q6.clone(), tds, ph, 64, PHASE_DECODE)
 
 

@@ -34,7 +34,7 @@ uint64_t decode_slots(int B, int G, int nw) { return (uint64_t)nw + (uint64_t)B 
 // slots bring fewer workgroups than the chip has CUs splits the keys of every item; 0 = the shape never splits.
 constexpr int kPrefillFillWorkgroups = 256;
 constexpr int kPrefillMaxSplitSlots = 64;
-int prefill_rows_per_workgroup(int D) { return D > 256 ? 64 : 128; }
+int prefill_rows_per_workgroup(int /*D*/) { return 128; }
 int prefill_split_slots(int H, int G, int Tq, int D) {
     const int R = H / G, bm = prefill_rows_per_workgroup(D);
     if (R < 1 || bm % R) return 0;

@@ -11,7 +11,7 @@ namespace g4b {
 hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
 // any Tq; (H/G) must divide 128; D in {128, 256}
 hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
-// any Tq; (H/G) must divide 64; D = 512
+// any Tq; (H/G) must divide 128; D = 512
 hipError_t launch_attn_prefill_wide(const AttnParams& p, int kv_dt, hipStream_t stream);
 
 struct KvAppendParams {

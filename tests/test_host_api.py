@@ -115,9 +115,9 @@ def test_python_boundary_validates_like_the_reference(native):
     q5, k5 = torch.zeros(2, 8, 1, 192, dtype=torch.float16), torch.zeros(2, 2, 64, 192, dtype=torch.float16)
     with pytest.raises(NotImplementedError, match="head_dim"):
         flash_attention(q5, k5, k5, q5.clone(), tds, ph, 64, PHASE_DECODE)
-    # prefill-shaped launches: the group size must divide the rows of a workgroup (64 for head dimension 512)
+    # prefill-shaped launches: the group size must divide the rows of a workgroup (128)
     q6, k6 = torch.zeros(2, 6, 8, 512, dtype=torch.float16), torch.zeros(2, 2, 64, 512, dtype=torch.float16)
-    with pytest.raises(NotImplementedError, match="must divide 64"):
+    with pytest.raises(NotImplementedError, match="must divide 128"):
         flash_attention(q6, k6, k6, q6.clone(), tds, ph, 64, PHASE_DECODE)
 
 

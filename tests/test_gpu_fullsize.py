@@ -28,7 +28,7 @@ def oracle_rows(q, k, v, b, rows, tds, W, Tq, stage=ix.STAGE_CAUSAL, qw=None):
     idx = (torch.arange(win, device=k.device) + start) % kv_ctx
     kl = k[b][:, idx].double().cpu().numpy()
     vl = v[b][:, idx].double().cpu().numpy()
-    out = np.zeros((H, len(rows), D))
+    out = np.zeros((H, len(rows), q.shape[-1]))
     for n, i in enumerate(rows):
         lo, hi = ix.visible_range(i, tds, W, Tq, stage, qw)
         for h in range(H):
@@ -141,6 +141,40 @@ def test_config3_uniform_attention_is_the_running_mean(fa):
     lo = (idx - 511).clamp(min=0)
     wmean = (cs[:, idx + 1] - cs[:, lo]) / (idx + 1 - lo).double()[None, :, None]
     assert_close(o[0].cpu().numpy(), wmean.repeat_interleave(H // G, 0).cpu().numpy(), atol=1e-3, rtol=1e-3, what="windowed mean")
+
+
+def test_head_dim_512_prefill_8192_and_decode_batch(fa):
+    """Head dimension 512 (the global-attention layers) at the sizes of configurations 3 and 4: sampled rows against the
+    oracle, uniform attention as the running mean, split against unsplit decode."""
+    S, D5 = 8192, 512
+    q, k, v = randn16((1, H, S, D5), 1), randn16((1, G, S, D5), 2), randn16((1, G, S, D5), 3)
+    o = torch.full_like(q, 777.0)
+    fa.flash_attention(q, k, v, o, i32([S]), u8([1]), S, 1, scale=SCALE)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    rows = [0, 1, 31, 32, 127, 128, 4095, 4096, 8190, 8191] + np.random.default_rng(2).integers(0, S, 10).tolist()
+    assert_close(got[0][:, rows], oracle_rows(q, k, v, 0, rows, S, S, S), what="D=512 prefill 8192")
+    o32 = torch.empty(1, H, S, D5, device="cuda", dtype=torch.float32)
+    fa.flash_attention(q, torch.zeros_like(k), v, o32, i32([S]), u8([1]), S, 1, scale=SCALE)
+    torch.cuda.synchronize()
+    mean = v[0].double().cumsum(1) / torch.arange(1, S + 1, device="cuda").double()[None, :, None]
+    assert_close(o32[0].cpu().numpy(), mean.repeat_interleave(H // G, 0).cpu().numpy(), atol=1e-3, rtol=1e-3, what="running mean")
+    del q, k, v, o, o32
+    B, kv_ctx = 32, 32768
+    tds = np.random.default_rng(3).integers(128, kv_ctx + 1, B).tolist()
+    q, k, v = randn16((B, H, 1, D5), 1), randn16((B, G, kv_ctx, D5), 2), randn16((B, G, kv_ctx, D5), 3)
+    o = torch.full_like(q, 777.0)
+    ws = torch.empty(fa.workspace_bytes(B, H, G, 1, D5), dtype=torch.uint8, device="cuda")
+    fa.flash_attention(q, k, v, o, i32(tds), u8([2] * B), kv_ctx, 2, scale=SCALE, workspace=ws)
+    o1 = torch.empty_like(q)
+    fa.flash_attention(q, k, v, o1, i32(tds), u8([2] * B), kv_ctx, 2, scale=SCALE)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    for b in [0, 5, 31, int(np.argmax(tds)), int(np.argmin(tds))]:
+        assert_close(got[b], oracle_rows(q, k, v, b, [0], tds[b], kv_ctx, 1), what=f"D=512 decode slot {b}")
+    d = (o1.float() - o.float()).abs()
+    assert bool((d <= 5e-4 + 2e-3 * o.float().abs()).all()), d.max().item()
 
 
 def test_config2_causal_prefill_2048_all_rows(fa):

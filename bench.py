@@ -41,6 +41,8 @@ FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PMC_TRAFFIC_KIB = {
     "decode_batched_b64": {"fetch": 579346.1, "write": 4544.8},
     "prefill_causal_8192": {"fetch": 82093.4, "write": 32768.0},
+    "decode_batched_b32_d512": {"fetch": 1110179.4, "write": 4589.9},
+    "prefill_causal_8192_d512": {"fetch": 239551.2, "write": 65536.0},
 }
 PMC_SCALE = {"fetch": 2.000, "write": 1.000}
 

@@ -158,11 +158,11 @@ def test_prefill_key_split_agrees_with_one_workgroup_per_tile(fa, case):
     assert bool((diff <= 5e-4 + 2e-3 * o.float().abs()).all()), diff.max().item()
 
 
-@pytest.mark.parametrize("n_prefill", [1, 2, 5, 9])
-def test_prefill_chunk_inside_a_mixed_batch(fa, n_prefill):
+@pytest.mark.parametrize("n_prefill,D", [(1, 256), (2, 256), (5, 256), (9, 256), (1, 512), (3, 512), (9, 512)])
+def test_prefill_chunk_inside_a_mixed_batch(fa, n_prefill, D):
     """The engine's mixed step: a few slots prefill a chunk while the others decode or are unallocated.  The number of
     key splits follows the number of in-phase slots, which only the device knows."""
-    B, H, G, Tq, D, W = 9, 8, 2, 96, 256, 3000
+    B, H, G, Tq, W = 9, 8, 2, 96, 3000
     kv_ctx = W + Tq - 1
     q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=15)
     order = [4, 0, 8, 2, 6, 1, 3, 5, 7]
@@ -225,10 +225,10 @@ def test_one_shot_causal_prefill_2048(fa):
     assert_close(o.float().cpu().numpy(), ref, what="config 2")
 
 
-@pytest.mark.parametrize("qw", [1, 37, 64, 512, 5000])
-def test_per_query_sliding_window(fa, qw):
+@pytest.mark.parametrize("qw,D", [(1, 256), (37, 256), (64, 256), (512, 256), (5000, 256), (1, 512), (37, 512), (500, 512)])
+def test_per_query_sliding_window(fa, qw, D):
     """One-shot prefill longer than the window: key visible iff 0 <= q_pos - k_pos < query_window."""
-    B, H, G, Tq, D = 1, 8, 2, 1024, 256
+    B, H, G, Tq = 1, 8, 2, 1024
     q, k, v, o = make_case(B, H, G, Tq, D, Tq, seed=5)
     ref = oracle(q, k, v, [Tq], [1], Tq, 1, scale=1 / 16, query_window=qw)
     fa.flash_attention(q, k, v, o, i32([Tq]), u8([1]), Tq, 1, scale=1 / 16, query_window=qw)
@@ -236,9 +236,10 @@ def test_per_query_sliding_window(fa, qw):
     assert_close(o.float().cpu().numpy(), ref, what=f"query_window={qw}")
 
 
-def test_chunk_on_long_context_with_wrap(fa):
+@pytest.mark.parametrize("D", [256, 512])
+def test_chunk_on_long_context_with_wrap(fa, D):
     """A 512-token chunk appended to an existing context in a ring of W + t - 1 rows (gemma4e.py:703-705)."""
-    B, H, G, t, D, W = 2, 8, 2, 512, 256, 2048
+    B, H, G, t, W = 2, 8, 2, 512, 2048
     kv_ctx = W + t - 1
     q, k, v, o = make_case(B, H, G, t, D, kv_ctx, seed=6)
     tds = [1500 + t, 9000 + t]  # second slot: window full, ring wrapped several times
@@ -287,9 +288,10 @@ def test_engine_layout_fp32_strided_views(fa, Tq):
     assert_close(o.cpu().numpy(), ref, what="engine layout")
 
 
+@pytest.mark.parametrize("D", [256, 512])
 @pytest.mark.parametrize("Tq", [1, 160])
-def test_bf16_cache(fa, Tq):
-    B, H, G, D, W = 2, 8, 2, 256, 1024
+def test_bf16_cache(fa, Tq, D):
+    B, H, G, W = 2, 8, 2, 1024
     q, k, v, o = make_case(B, H, G, Tq, D, W, seed=9, dtype=torch.bfloat16)
     tds = [W, W + 17]
     phase_id = 2 if Tq == 1 else 1
@@ -300,11 +302,12 @@ def test_bf16_cache(fa, Tq):
     assert_close(o.float().cpu().numpy(), ref, atol=ATOL_BF16, rtol=RTOL_BF16, what="bf16")
 
 
+@pytest.mark.parametrize("D", [256, 512])
 @pytest.mark.parametrize("Tq", [1, 4, 40])
-def test_visible_set_is_bit_exact(fa, Tq):
+def test_visible_set_is_bit_exact(fa, Tq, D):
     """K = 0 makes the weights uniform; V row r = e_(r mod D) turns the output into the indicator of the
     ring rows that were read divided by their count, so the visible set is read back exactly."""
-    B, H, G, D = 4, 8, 2, 256
+    B, H, G = 4, 8, 2
     kv_ctx, W = 251, 200  # W <= KV_CTX <= D so that every ring row has its own output column
     q = torch.randn(B, H, Tq, D, device="cuda").half()
     k = torch.zeros(B, G, kv_ctx, D, device="cuda", dtype=torch.float16)

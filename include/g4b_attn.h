@@ -28,7 +28,7 @@ extern "C" {
 enum g4b_status {
     G4B_OK = 0,
     G4B_ERR_INVALID_ARGUMENT = -1, /* shape / stride / dtype / value check failed (reference: tl.static_assert) */
-    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim 512 with more than 16 query rows per kv head, STAGE_ON_BAND alone) */
+    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim 64, STAGE_ON_BAND alone) */
     G4B_ERR_WORKSPACE = -3,        /* workspace missing or too small for the requested split-KV launch */
     G4B_ERR_LAUNCH = -4            /* the HIP runtime refused the launch (no device, bad stream, ...) */
 };
@@ -65,8 +65,9 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *                 and a prefill-shaped launch one workgroup per (slot, kv head, query tile) however
  *                 few slots are in phase.  Contents are unspecified after the call (like
  *                 partial_o/l/m, fa2.py:643-645).
- *   num_workers   0 = library default; otherwise the number of waves the decode key tiles are
- *                 dealt to (must not exceed the value the workspace was sized for).  Ignored by
+ *   num_workers   0 = library default; otherwise the number of workers the decode key tiles are
+ *                 dealt to (must not exceed the value the workspace was sized for).  A worker is one
+ *                 wave, or a pair of waves when D = 512.  Ignored by
  *                 prefill-shaped launches, which choose their key split from the number of in-phase
  *                 slots on the device.
  *   kernel_mask   profiling aid.  0 = run every kernel of the launch.  Otherwise bit 0 selects the
@@ -109,13 +110,14 @@ typedef struct g4b_attn_args {
 int g4b_attn_forward(const g4b_attn_args* args, void* stream);
 
 /* Bytes of workspace that let g4b_attn_forward split keys: for a decode-shaped launch (R*Tq <= 16)
- * over `num_workers` waves (0 = library default); for a prefill shape that brings fewer workgroups
+ * over `num_workers` workers (0 = library default); for a prefill shape that brings fewer workgroups
  * per slot than the chip has compute units (chunked prefill, short prompts; sized by H, G, Tq, D
  * only) over several workgroups per query tile.  Returns 0 when the shape never uses a workspace.
  * Replaces the sizing of partial_o/l/m at g4b/models/gemma4e.py:43,819-821. */
 uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers);
 
-/* The library default for num_workers on the current build (a multiple of the CU count). */
+/* The library default for num_workers on the current build (a multiple of the CU count) for D <= 256;
+ * half of it for D = 512, whose workers are pairs of waves. */
 int32_t g4b_attn_default_workers(void);
 
 /*

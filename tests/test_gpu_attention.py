@@ -288,6 +288,23 @@ def test_engine_layout_fp32_strided_views(fa, Tq):
     assert_close(o.cpu().numpy(), ref, what="engine layout")
 
 
+@pytest.mark.parametrize("Tq,D", [(1, 256), (96, 256), (1, 512), (96, 512)])
+def test_fp16_output_straight_into_the_token_major_activation_buffer(fa, Tq, D):
+    """fp32 q scratchpad in, fp16 o out, o being the [B, t, H*D] buffer the next matmul reads: no cast or layout pass
+    between the kernels (the reference keeps both sides fp32 and casts afterwards, gemma4e.py:1031-1033)."""
+    B, H, G, W = 3, 8, 2, 700
+    q, k, v, _ = make_case(B, H, G, Tq, D, W, seed=18, q_dtype=torch.float32, engine_layout=True)
+    act = torch.full((B, Tq, H * D), 777.0, dtype=torch.float16, device="cuda")
+    o = act.view(B, Tq, H, D).permute(0, 2, 1, 3)
+    tds = [W, W + 17, max(Tq, 5)]
+    phase_id = 2 if Tq == 1 else 1
+    ref = oracle(q.half(), k, v, tds, [phase_id] * B, W, phase_id, scale=0.0625)
+    fa.flash_attention(q, k, v, o, i32(tds), u8([phase_id] * B), W, phase_id, scale=0.0625)
+    torch.cuda.synchronize()
+    got = act.view(B, Tq, H, D).permute(0, 2, 1, 3).float().cpu().numpy()
+    assert_close(got, ref, what="fp16 o in [B,t,H*D]")
+
+
 @pytest.mark.parametrize("D", [256, 512])
 @pytest.mark.parametrize("Tq", [1, 160])
 def test_bf16_cache(fa, Tq, D):

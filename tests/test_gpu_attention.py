@@ -183,6 +183,45 @@ def test_prefill_chunk_inside_a_mixed_batch(fa, n_prefill, D):
             assert (got[b] == 123.0).all(), f"off-phase slot {b} was written"
 
 
+@pytest.mark.parametrize("D", [256, 512])
+def test_more_than_64_slots(fa, D):
+    """Batches beyond one wavefront of slots: the device-side work lists walk the slots 64 (decode) or 256 (prefill
+    shapes) at a time.  150 slots with ragged lengths; decode over the odd slots, then a 40-token chunk on five slots
+    scattered over the batch."""
+    B, H, G, W = 150, 8, 2, 96
+    rng = np.random.default_rng(41)
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=41)
+    tds = rng.integers(0, 2 * W, B).tolist()
+    phase = [2 if b % 2 else 0 for b in range(B)]
+    ref = oracle(q, k, v, tds, phase, W, 2, scale=1 / 16)
+    for parts in ((), partials(4, B, H, 1, D)):
+        o.fill_(123.0)
+        fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 2, *parts, scale=1 / 16)
+        torch.cuda.synchronize()
+        got = o.float().cpu().numpy()
+        for b in range(B):
+            if phase[b] == 2:
+                assert_close(got[b], ref[b], what=f"decode slot {b} split={bool(parts)}")
+            else:
+                assert (got[b] == 123.0).all(), f"off-phase slot {b} was written"
+    Tq = 40
+    kv_ctx = W + Tq - 1
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=42)
+    chunking = [3, 64, 65, 128, 149]
+    phase = [1 if b in chunking else 2 for b in range(B)]
+    tds = [Tq + int(x) for x in rng.integers(0, 3 * W, B)]
+    ref = oracle(q, k, v, tds, phase, W, 1, scale=1 / 16)
+    o.fill_(123.0)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, scale=1 / 16)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(got[b], ref[b], what=f"chunk on slot {b}")
+        else:
+            assert (got[b] == 123.0).all(), f"off-phase slot {b} was written"
+
+
 def test_prefill_workspace_too_small_is_refused(fa):
     B, H, G, Tq, D, W = 1, 8, 2, 128, 256, 1024
     q, k, v, o = make_case(B, H, G, Tq, D, W, seed=16)

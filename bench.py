@@ -56,6 +56,17 @@ H, G, D = 8, 2, 256
 SCALE = 1.0 / 16.0
 
 
+def host_cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -478,7 +489,8 @@ def main():
             secs, done, desc = wl.cpu_sample()
             unit, val = ("GB/s", done / secs / 1e9) if wl.bound == "hbm" else ("TFLOP/s", done / secs / 1e12)
             cpu = {"value": round(val, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
-                   "sample": f"{desc}; {secs:.2f} s; torch CPU fp32 restatement of scripts/reference_impl.py:421-443"}
+                   "sample": f"{desc}; {secs:.2f} s; torch CPU fp32 restatement of scripts/reference_impl.py:421-443",
+                   "cpu_model": host_cpu_model()}
             log(f"cpu baseline: {cpu}")
         except NotImplementedError:
             cpu = None

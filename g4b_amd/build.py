@@ -2,6 +2,7 @@
 
     python -m g4b_amd.build            # compile every translation unit, link
     python -m g4b_amd.build --verbose  # also print the per-kernel register / LDS usage remarks
+    python -m g4b_amd.build --check-waits  # also verify that nothing foreign sits in the hand-counted wait regions
 
 The shared library lands next to this file so that it travels with the source tree; nothing
 is installed.  hipcc cross-compiles for gfx950 without a GPU present.
@@ -65,6 +66,53 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     return LIB_PATH
 
 
+# Kernels whose LDS operand reads are retired with hand-counted `s_waitcnt lgkmcnt(n)` and whose direct-to-LDS loads
+# are waited for with one `s_waitcnt vmcnt(0)` per tile.  The counts are only exact while the compiler keeps its own
+# memory traffic out of the region between the first and the last MFMA: a scalar load or a compiler-made LDS access
+# there shares lgkmcnt (and scalar loads return out of order), a global or scratch access brings a vmcnt(0) that also
+# waits for the direct loads in flight.
+PIPELINED_SOURCES = {"attn_prefill.hip": "attn_prefill_kernel", "attn_prefill_wide.hip": "attn_prefill_wide_kernel"}
+
+
+def check_wait_discipline() -> dict:
+    """Compile the pipelined kernels to assembly and scan the MFMA region of each instantiation.
+
+    Returns {kernel symbol: number of MFMAs}; raises RuntimeError naming the first foreign memory instruction."""
+    import re
+    import tempfile
+
+    foreign = re.compile(r"\b(s_load|s_buffer_load|scratch_|global_load_dword|global_store|buffer_|flat_|ds_)")
+    allowed = ("ds_read_b128", "ds_read_b64_tr_b16", "global_load_lds_dwordx4")
+    seen = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        for src, stem in PIPELINED_SOURCES.items():
+            out = Path(tmp) / (src + ".s")
+            cmd = [hipcc(), *COMMON_FLAGS, *DEVICE_FLAGS, "-S", "--cuda-device-only", str(CSRC / src), "-o", str(out)]
+            res = subprocess.run(cmd, capture_output=True, text=True)
+            if res.returncode != 0:
+                raise RuntimeError(f"hipcc -S failed on {src}:\n{res.stderr}")
+            lines = out.read_text().splitlines()
+            i = 0
+            while i < len(lines):
+                m = re.match(r"(_ZN3g4b\d+%s\w*):" % stem, lines[i])
+                if not m:
+                    i += 1
+                    continue
+                end = next(j for j in range(i, len(lines)) if lines[j].startswith(".Lfunc_end"))
+                body = lines[i:end]
+                mfma = [j for j, l in enumerate(body) if "v_mfma" in l]
+                for l in body[mfma[0] : mfma[-1] + 1]:
+                    ins = l.strip()
+                    if foreign.search(ins) and not ins.startswith(allowed):
+                        raise RuntimeError(f"{m.group(1)}: `{ins}` inside the hand-counted wait region")
+                seen[m.group(1)] = len(mfma)
+                i = end
+    return seen
+
+
 if __name__ == "__main__":
     path = build(verbose="--verbose" in sys.argv)
     print(path)
+    if "--check-waits" in sys.argv:
+        for sym, n in check_wait_discipline().items():
+            print(f"wait discipline ok: {sym} ({n} MFMAs)")

@@ -197,3 +197,14 @@ def test_plan_validates_at_bind_time(native):
     bad = plan_flash_attention(q, k, v, o, tds, ph, 65, PHASE_DECODE)
     with pytest.raises(ValueError, match="ctx_window_size"):  # value checks live in the library (fa2.py:298)
         bad.launch(stream=0)
+
+
+def test_pipelined_kernels_keep_foreign_memory_traffic_out_of_their_wait_regions():
+    """The prefill kernels retire LDS reads with hand-counted lgkmcnt waits and direct-to-LDS loads with one vmcnt(0)
+    per tile; a compiler-made scalar, LDS, global or scratch access between the first and the last MFMA would break
+    the counts (a spill is enough).  The build module scans the generated assembly."""
+    from g4b_amd.build import check_wait_discipline
+
+    seen = check_wait_discipline()
+    assert len(seen) == 6, seen  # head dims 128 and 256 in fp16 and bf16, head dim 512 in fp16 and bf16
+    assert all(n >= 48 for n in seen.values()), seen

@@ -7,7 +7,8 @@
 // time_dim_sizes, so the grid is static while the balance follows the real lengths.  A worker
 // whose range covers a whole pair writes the output directly; otherwise it leaves an
 // un-normalised fp32 partial (acc, running max, running sum) in workspace slot (w + pair) and a
-// second kernel merges the partials of each pair.
+// second kernel merges the partials of each pair.  Launches whose window is at most 512 keys take a one-kernel
+// variant instead (attn_decode_pair: four waves per pair, merged through LDS).
 //
 // Tile math (one wave, 32 keys).  S^T = K Q^T and O^T += V^T P run on v_mfma_f32_16x16x32.
 // The 16 output columns carry (row, class) pairs: the D/8 16-byte pieces of a key row are dealt
@@ -48,8 +49,12 @@ G4B_DEV float pick(const f4& c, int e, int cls) {
 // DH > 1: the workgroup has DH waves and wave hv owns columns [hv*D/DH, (hv+1)*D/DH) of the head dimension: its share
 // of q, of every K and V row and of the output.  The waves add their partial dot products through LDS once per tile
 // and then run the same softmax, so the register tiling is that of head dimension D/DH.
+//
+// lds_part != nullptr: the un-normalised result goes to that LDS block ([16 rows][D] floats, then [16 rows][2] of
+// (reference, sum)) whatever the segment covers; the caller merges the blocks of its waves.
 template <int D, int CL, class T, int DH>
-G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb, float* xch) {
+G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb, float* xch,
+                            float* lds_part = nullptr) {
     constexpr int DL = D / DH;         // columns this wave owns
     constexpr int E = 4 / CL;          // scores a lane keeps per 16-row MFMA tile
     constexpr int KT = 16 / CL;        // keys per MFMA tile
@@ -208,7 +213,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
     // ---- epilogue -----------------------------------------------------------------
     float l_tot = l_run + __shfl_xor(l_run, 16);
     l_tot += __shfl_xor(l_tot, 32);
-    const bool whole = (t0 == 0 && t1 == tlb);
+    const bool whole = (t0 == 0 && t1 == tlb) && lds_part == nullptr;
     if (row_ok) {
         if (whole) {
             const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
@@ -227,7 +232,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
             }
         } else {
             const int64_t slot = (int64_t)w + (int64_t)bb * G + g;
-            float* po = p.part_o + (slot * NR + row) * D;
+            float* po = lds_part ? lds_part + row * D : p.part_o + (slot * NR + row) * D;
 #pragma unroll
             for (int dc = 0; dc < DC; ++dc) {
 #pragma unroll
@@ -240,7 +245,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
                 }
             }
             if (cls == 0 && g4 == 0 && hv == 0) {
-                float* pm = p.part_ml + (slot * NR + row) * 2;
+                float* pm = lds_part ? lds_part + 16 * D + row * 2 : p.part_ml + (slot * NR + row) * 2;
                 pm[0] = m_run;
                 pm[1] = l_tot;
             }
@@ -300,6 +305,59 @@ __global__ __launch_bounds__(64 * DH, 1) void attn_decode_worker(const AttnParam
         }
         carry += __shfl(incl, 63);
         if ((int64_t)carry >= we) break;
+    }
+}
+
+// Short windows (a sliding-window layer: at most a few dozen tiles per pair): one workgroup of four waves per (slot, kv
+// head) pair, each wave a quarter of the pair's tiles, merged through LDS in the same launch.  With so little work per
+// pair the two-kernel path is all latency (worker prologue, partials out and back in, second launch).
+constexpr int DEC_PAIR_WAVES = 4;
+template <int D>
+constexpr int dec_pair_smem() { return DEC_PAIR_WAVES * (16 * D + 32) * (int)sizeof(float); }
+
+template <int D, int CL, class T>
+__global__ __launch_bounds__(64 * DEC_PAIR_WAVES, 1) void attn_decode_pair(const AttnParams p) {
+    extern __shared__ __align__(16) float pair_smem[];
+    constexpr int BLK = 16 * D + 32;  // floats per wave block
+    const int tid = threadIdx.x, wave = tid >> 6;
+    const int pair = blockIdx.x;
+    const int bb = pair / p.G, g = pair % p.G;
+    const SlotInfo si = slot_info(p, bb);
+    if (!si.active) return;
+    const int NR = p.R * p.Tq;
+    const int tl = slot_tiles(p, bb);
+    float* mine = pair_smem + wave * BLK;
+    const int t0 = wave * tl / DEC_PAIR_WAVES, t1 = (wave + 1) * tl / DEC_PAIR_WAVES;
+    if (t1 > t0) {
+        decode_segment<D, CL, T, 1>(p, 0, bb, g, t0, t1, tl, nullptr, mine);
+    } else if ((tid & 63) < 16) {
+        mine[16 * D + (tid & 63) * 2] = -INFINITY;  // this wave brought no keys
+        mine[16 * D + (tid & 63) * 2 + 1] = 0.f;
+    }
+    __syncthreads();
+    // merge: a thread per four output columns of a row
+    constexpr int LPR = D / 4;
+    for (int item = tid; item < NR * LPR; item += 64 * DEC_PAIR_WAVES) {
+        const int row = item / LPR, c4 = item % LPR;
+        float mref = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_PAIR_WAVES; ++w) mref = fmaxf(mref, pair_smem[w * BLK + 16 * D + row * 2]);
+        const float msafe = (mref == -INFINITY) ? 0.f : mref;
+        f4 acc = {0.f, 0.f, 0.f, 0.f};
+        float l = 0.f;
+#pragma unroll
+        for (int w = 0; w < DEC_PAIR_WAVES; ++w) {
+            const float m = pair_smem[w * BLK + 16 * D + row * 2];
+            if (m != -INFINITY) {
+                const float e = fast_exp2(m - msafe);
+                acc += *reinterpret_cast<const f4*>(pair_smem + w * BLK + row * D + c4 * 4) * e;
+                l += pair_smem[w * BLK + 16 * D + row * 2 + 1] * e;
+            }
+        }
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        const int64_t ooff =
+            (int64_t)bb * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] + (int64_t)(row % p.Tq) * p.o_s[2];
+        store4(p.o, ooff + c4 * 4, p.o_dt, acc * inv);
     }
 }
 
@@ -404,8 +462,31 @@ __global__ __launch_bounds__(256) void attn_decode_combine(const AttnParams p) {
     }
 }
 
+// Host-side choice (static in the launch arguments, so a recorded graph keeps it): the one-kernel path when no slot
+// can bring more than DEC_PAIR_MAX_KEYS keys (four tiles per wave; beyond that the waves' sequential tiles cost more
+// than the second launch saves).
+constexpr int DEC_PAIR_MAX_KEYS = 512;
+static bool decode_pair_path(const AttnParams& p, int D) {
+    return D <= 256 && p.win_arr == nullptr && (p.W < p.KV_CTX ? p.W : p.KV_CTX) <= DEC_PAIR_MAX_KEYS;
+}
+
 template <int D, int CL, class T>
 static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
+    if constexpr (D <= 256) {
+        if (decode_pair_path(p, D)) {
+            static bool attr_set = false;
+            if (!attr_set) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_decode_pair<D, CL, T>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, dec_pair_smem<D>());
+                if (e != hipSuccess) return e;
+                attr_set = true;
+            }
+            if (p.kernel_mask & 1)
+                hipLaunchKernelGGL((attn_decode_pair<D, CL, T>), dim3(p.B * p.G), dim3(64 * DEC_PAIR_WAVES), dec_pair_smem<D>(),
+                                   stream, p);
+            return hipGetLastError();
+        }
+    }
     constexpr int DH = D > 256 ? D / 256 : 1;  // waves per worker: each owns at most 256 columns
     if (p.kernel_mask & 1) {
         hipLaunchKernelGGL((attn_decode_worker<D, CL, T, DH>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64 * DH), 0, stream,

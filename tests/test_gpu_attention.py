@@ -183,6 +183,36 @@ def test_prefill_chunk_inside_a_mixed_batch(fa, n_prefill, D):
             assert (got[b] == 123.0).all(), f"off-phase slot {b} was written"
 
 
+@pytest.mark.parametrize("Tq,H,G,D", [(1, 8, 2, 256), (1, 16, 2, 128), (3, 8, 2, 256), (1, 16, 1, 256)])
+def test_short_window_one_kernel_path_agrees_with_the_two_kernel_path(fa, Tq, H, G, D):
+    """Windows of at most 512 keys (the sliding-window layers) run as one launch that merges a pair's waves through
+    LDS; passing the same window per slot through window_sizes takes the worker + merge kernels instead.  Ragged
+    lengths from 0 keys to a wrapped ring; both against the oracle and against each other."""
+    B, W = 11, 512
+    kv_ctx = W + 5
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=51)
+    tds = [Tq, Tq + 1, 31 + Tq, 32 + Tq, 33 + Tq, 128, 129, 500, 512, 513, 5000]
+    phase = [1 if Tq > 1 else 2] * B
+    phase[4] = 0
+    ph = phase[0]
+    ref = oracle(q, k, v, tds, phase, W, ph, scale=1 / 16)
+    o.fill_(321.0)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), W, ph, *partials(4, B, H, Tq, D), scale=1 / 16)
+    o2 = torch.full_like(o, 321.0)
+    fa.flash_attention(q, k, v, o2, i32(tds), u8(phase), W, ph, *partials(4, B, H, Tq, D), scale=1 / 16,
+                       window_sizes=i32([W] * B))
+    torch.cuda.synchronize()
+    got, got2 = o.float().cpu().numpy(), o2.float().cpu().numpy()
+    for b in range(B):
+        if phase[b] == 0:
+            assert (got[b] == 321.0).all() and (got2[b] == 321.0).all()
+        else:
+            assert_close(got[b], ref[b], what=f"one-kernel path slot {b}")
+            assert_close(got2[b], ref[b], what=f"two-kernel path slot {b}")
+    d = np.abs(got - got2)
+    assert (d <= 5e-4 + 2e-3 * np.abs(got2)).all(), d.max()
+
+
 @pytest.mark.parametrize("D", [256, 512])
 def test_more_than_64_slots(fa, D):
     """Batches beyond one wavefront of slots: the device-side work lists walk the slots 64 (decode) or 256 (prefill

@@ -64,7 +64,8 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *                 NULL: then a decode-shaped launch (R*Tq <= 16) uses one wave per (slot, kv head)
  *                 and a prefill-shaped launch one workgroup per (slot, kv head, query tile) however
  *                 few slots are in phase.  Contents are unspecified after the call (like
- *                 partial_o/l/m, fa2.py:643-645).
+ *                 partial_o/l/m, fa2.py:643-645).  A decode-shaped launch with D <= 256,
+ *                 ctx_window_size <= 512 and no window_sizes merges in LDS and never touches it.
  *   num_workers   0 = library default; otherwise the number of workers the decode key tiles are
  *                 dealt to (must not exceed the value the workspace was sized for).  A worker is one
  *                 wave, or a pair of waves when D = 512.  Ignored by

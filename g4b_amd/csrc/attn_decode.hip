@@ -474,13 +474,9 @@ template <int D, int CL, class T>
 static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
     if constexpr (D <= 256) {
         if (decode_pair_path(p, D)) {
-            static bool attr_set = false;
-            if (!attr_set) {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_decode_pair<D, CL, T>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, dec_pair_smem<D>());
-                if (e != hipSuccess) return e;
-                attr_set = true;
-            }
+            static uint64_t attr_done = 0;
+            hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_decode_pair<D, CL, T>), dec_pair_smem<D>(), attr_done);
+            if (e != hipSuccess) return e;
             if (p.kernel_mask & 1)
                 hipLaunchKernelGGL((attn_decode_pair<D, CL, T>), dim3(p.B * p.G), dim3(64 * DEC_PAIR_WAVES), dec_pair_smem<D>(),
                                    stream, p);

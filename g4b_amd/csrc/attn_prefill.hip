@@ -470,13 +470,9 @@ static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     const int blocks = prefill_grid(p);
     dim3 grid(blocks);
     const int smem = 4 * PfSmem<D>::TILE;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static uint64_t attr_done = 0;
+    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T>), smem, attr_done);
+    if (e != hipSuccess) return e;
     if (p.kernel_mask & 1) hipLaunchKernelGGL((attn_prefill_kernel<D, T>), grid, dim3(256), smem, stream, p);
     if (slots > 1 && (p.kernel_mask & 2)) {
         const int items = min(p.B, slots / 2);  // more active slots than this are never split

@@ -353,13 +353,9 @@ template <class T>
 static hipError_t launch_prefill_wide_t(const AttnParams& p, hipStream_t stream) {
     const int slots = p.part_o ? p.split_slots : 1;
     const int blocks = prefill_grid(p, PW_BM);
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<T>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, PW_SMEM);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static uint64_t attr_done = 0;
+    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<T>), PW_SMEM, attr_done);
+    if (e != hipSuccess) return e;
     if (p.kernel_mask & 1) hipLaunchKernelGGL((attn_prefill_wide_kernel<T>), dim3(blocks), dim3(256), PW_SMEM, stream, p);
     if (slots > 1 && (p.kernel_mask & 2)) {
         const int items = min(p.B, slots / 2);  // more active slots than this are never split

@@ -7,6 +7,18 @@
 
 namespace g4b {
 
+// Raise a kernel's dynamic shared memory limit once per device (the attribute belongs to the function on the current
+// device).  `done` is the call site's bit mask of devices already served.
+inline hipError_t allow_dynamic_smem(const void* kernel, int bytes, uint64_t& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && ((done >> dev) & 1)) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && dev >= 0 && dev < 64) done |= 1ull << dev;
+    return e;
+}
+
 // rows = (H/G) * Tq <= 16, D in {128, 256, 512}; kv_dt in {DT_F16, DT_BF16}
 hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
 // any Tq; (H/G) must divide 128; D in {128, 256}

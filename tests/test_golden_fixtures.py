@@ -53,13 +53,15 @@ def test_kernels_match_fixture(gpu_device, path, split):
     t = lambda name: torch.from_numpy(f[name]).to(gpu_device)
     q, k, v = t("q"), t("k_cache"), t("v_cache")
     B, H, Tq, D = q.shape
-    if split and (H // k.shape[1]) * Tq > 16:
-        pytest.skip("split buffers only matter for decode-shaped launches")
     o = torch.full((B, H, Tq, D), 777.0, dtype=torch.float16, device=gpu_device)
-    parts = partials(4, B, H, Tq, D) if split else ()
+    decode_shaped = (H // k.shape[1]) * Tq <= 16
+    # decode-shaped launches split their keys when the partial buffers are passed; prefill-shaped ones split by
+    # themselves when the shape would underfill the chip unless workspace=False forbids it
+    parts = partials(4, B, H, Tq, D) if split and decode_shaped else ()
+    extra = {} if split or decode_shaped else {"workspace": False}
     flash_attention(
         q, k, v, o, t("time_dim_sizes"), t("user_phase"), int(f["ctx_window_size"]), int(f["phase"]), *parts,
-        stage=int(f["stage"]), scale=float(f["scale"]), query_window=int(f["query_window"]) or None,
+        stage=int(f["stage"]), scale=float(f["scale"]), query_window=int(f["query_window"]) or None, **extra,
     )
     torch.cuda.synchronize()
     assert_close(o.float().cpu().numpy(), f["expected"], what=os.path.basename(path))

@@ -148,6 +148,8 @@ EXPORTS = {
     "g4b_advance_decode_state": (C.c_int, [C.POINTER(AdvanceArgs), C.c_void_p]),
     "g4b_rope": (C.c_int, [C.POINTER(RopeArgs), C.c_void_p]),
     "g4b_rope_frequencies": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_float, C.c_void_p]),
+    "g4b_profile_begin": (C.c_int, []),
+    "g4b_profile_end": (C.c_int, [C.POINTER(C.c_float), C.c_int32]),
     "g4b_last_error": (C.c_char_p, []),
     "g4b_abi_version": (C.c_int32, []),
 }

@@ -5,12 +5,40 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <utility>
+#include <vector>
 
 #include "launch.hpp"
 
 namespace {
 
 thread_local char g_err[512] = "";
+
+// g4b_profile_begin .. g4b_profile_end: one (start, stop) event pair per timed call of this thread
+thread_local bool g_profiling = false;
+thread_local std::vector<std::pair<hipEvent_t, hipEvent_t>> g_profile_records;
+
+// Arm the events for the dominant kernel of the launcher call that follows; false if they cannot be created.
+bool profile_arm() {
+    if (!g_profiling) return true;
+    hipEvent_t a = nullptr, b = nullptr;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) {
+        if (a) (void)hipEventDestroy(a);
+        return false;
+    }
+    g_profile_records.emplace_back(a, b);
+    g4b::g_profile_events = g4b::ProfileEvents{a, b};
+    return true;
+}
+// After the launcher: events nobody consumed (the dominant kernel was masked out) mark an untimed call.
+void profile_disarm() {
+    if (g4b::g_profile_events.start) {
+        (void)hipEventDestroy(g_profile_records.back().first);
+        (void)hipEventDestroy(g_profile_records.back().second);
+        g_profile_records.back() = {nullptr, nullptr};
+        g4b::g_profile_events = g4b::ProfileEvents{};
+    }
+}
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -53,6 +81,38 @@ uint64_t prefill_workspace_bytes(int H, int G, int Tq, int D) {
 extern "C" {
 
 const char* g4b_last_error(void) { return g_err; }
+
+int g4b_profile_begin(void) {
+    if (g_profiling) return fail(G4B_ERR_INVALID_ARGUMENT, "g4b_profile_begin: already profiling on this thread");
+    g_profile_records.clear();
+    g_profiling = true;
+    return G4B_OK;
+}
+
+int g4b_profile_end(float* ms, int32_t capacity) {
+    if (!g_profiling) return fail(G4B_ERR_INVALID_ARGUMENT, "g4b_profile_end without g4b_profile_begin");
+    g_profiling = false;
+    int n = 0;
+    hipError_t first_err = hipSuccess;
+    for (auto& r : g_profile_records) {
+        float t = -1.f;
+        if (r.first) {
+            hipError_t e = hipEventSynchronize(r.second);
+            if (e == hipSuccess) e = hipEventElapsedTime(&t, r.first, r.second);
+            if (e != hipSuccess) {
+                t = -1.f;
+                if (first_err == hipSuccess) first_err = e;
+            }
+            (void)hipEventDestroy(r.first);
+            (void)hipEventDestroy(r.second);
+        }
+        if (ms && n < capacity) ms[n] = t;
+        ++n;
+    }
+    g_profile_records.clear();
+    if (first_err != hipSuccess) return fail(G4B_ERR_LAUNCH, "profiling events: %s", hipGetErrorString(first_err));
+    return n;
+}
 int32_t g4b_abi_version(void) { return G4B_ATTN_ABI_VERSION; }
 int32_t g4b_attn_default_workers(void) { return kDefaultWorkers; }
 
@@ -149,6 +209,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         } else {
             p.NW = 0;  // one wave per (slot, kv head), no partials
         }
+        if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
         const int bm = prefill_rows_per_workgroup(a->D);
@@ -165,9 +226,11 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
             p.part_o = static_cast<float*>(a->workspace);
             p.part_ml = p.part_o + (uint64_t)p.split_slots * a->H * a->Tq * a->D;
         }
+        if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = a->D == 512 ? g4b::launch_attn_prefill_wide(p, a->kv_dtype, static_cast<hipStream_t>(stream))
                         : g4b::launch_attn_prefill(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     }
+    profile_disarm();
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
     return G4B_OK;
 }
@@ -317,7 +380,9 @@ int g4b_rope(const g4b_rope_args* a, void* stream) {
     p.phase = a->phase;
     p.k_writeback = a->k_writeback;
     p.eps = a->rmsnorm_eps;
+    if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
     hipError_t e = g4b::launch_rope(p, static_cast<hipStream_t>(stream));
+    profile_disarm();
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "rope launch failed: %s", hipGetErrorString(e));
     return G4B_OK;
 }

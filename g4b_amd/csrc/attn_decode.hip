@@ -478,15 +478,15 @@ static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
             hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_decode_pair<D, CL, T>), dec_pair_smem<D>(), attr_done);
             if (e != hipSuccess) return e;
             if (p.kernel_mask & 1)
-                hipLaunchKernelGGL((attn_decode_pair<D, CL, T>), dim3(p.B * p.G), dim3(64 * DEC_PAIR_WAVES), dec_pair_smem<D>(),
-                                   stream, p);
+                G4B_LAUNCH_DOMINANT((attn_decode_pair<D, CL, T>), dim3(p.B * p.G), dim3(64 * DEC_PAIR_WAVES), dec_pair_smem<D>(),
+                                    stream, p);
             return hipGetLastError();
         }
     }
     constexpr int DH = D > 256 ? D / 256 : 1;  // waves per worker: each owns at most 256 columns
     if (p.kernel_mask & 1) {
-        hipLaunchKernelGGL((attn_decode_worker<D, CL, T, DH>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64 * DH), 0, stream,
-                           p);
+        G4B_LAUNCH_DOMINANT((attn_decode_worker<D, CL, T, DH>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64 * DH), 0, stream,
+                            p);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

@@ -1,11 +1,30 @@
 // Host-side launchers implemented by the kernel translation units.
 #pragma once
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include "common.hpp"
 
 namespace g4b {
+
+// Profiling aid: when the calling thread has armed a pair of events, the dominant kernel of the next launcher call is
+// dispatched with them (hipExtLaunchKernelGGL stamps the events with the begin and the end of that dispatch, so their
+// difference is the kernel's own duration, without the gaps an event pair recorded around the launch includes).
+struct ProfileEvents {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+inline thread_local ProfileEvents g_profile_events;
+#define G4B_LAUNCH_DOMINANT(kernel, grid, block, smem, stream, ...)                                                    \
+    do {                                                                                                               \
+        if (g4b::g_profile_events.start) {                                                                             \
+            hipExtLaunchKernelGGL(kernel, grid, block, smem, stream, g4b::g_profile_events.start,                      \
+                                  g4b::g_profile_events.stop, 0, __VA_ARGS__);                                         \
+            g4b::g_profile_events = g4b::ProfileEvents{};                                                              \
+        } else {                                                                                                       \
+            hipLaunchKernelGGL(kernel, grid, block, smem, stream, __VA_ARGS__);                                        \
+        }                                                                                                              \
+    } while (0)
 
 // Raise a kernel's dynamic shared memory limit once per device (the attribute belongs to the function on the current
 // device).  `done` is the call site's bit mask of devices already served.

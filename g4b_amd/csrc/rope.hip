@@ -175,7 +175,7 @@ hipError_t launch_rope(const RopeParams& p, hipStream_t stream) {
     int z = 1;
     while (z < 4 && z * 2 <= jobs && (int64_t)blocks * p.B * z < 256) z *= 2;
     dim3 grid(blocks, p.B, z);
-    hipLaunchKernelGGL(rope_kernel, grid, dim3(256), 0, stream, p);
+    G4B_LAUNCH_DOMINANT(rope_kernel, grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -231,6 +231,18 @@ int g4b_rope(const g4b_rope_args* args, void* stream);
 int g4b_rope_frequencies(float* out, const float* freq_scalars, int32_t n, int64_t out_stride,
                          int64_t freq_scalars_stride, float freq_base, void* stream);
 
+/*
+ * Profiling aid, no counterpart in the reference.  Between g4b_profile_begin() and g4b_profile_end() every
+ * g4b_attn_forward and g4b_rope call of the calling thread has its dominant kernel (the streaming worker, the prefill
+ * kernel, the rope kernel) dispatched with a pair of events that the runtime stamps with the begin and the end of that
+ * dispatch: the kernel's own duration, as a kernel trace reports it, without the launch gaps an event pair recorded
+ * around the call would include.  g4b_profile_end waits for the timed kernels, writes up to `capacity` durations in
+ * milliseconds in call order (-1 for a call whose dominant kernel was masked out) and returns the number of timed
+ * calls, or a negative g4b_status.  Events are created per call, so this is not for graph capture.
+ */
+int g4b_profile_begin(void);
+int g4b_profile_end(float* ms, int32_t capacity);
+
 /* Message of the calling thread's last failed call ("" if none). */
 const char* g4b_last_error(void);
 

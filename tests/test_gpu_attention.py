@@ -417,6 +417,40 @@ def test_visible_set_is_bit_exact(fa, Tq, D):
                     np.testing.assert_allclose(got[b, h, i, rows], 1.0 / len(rows), rtol=2e-3)
 
 
+def test_dispatch_stamped_kernel_times(fa):
+    """g4b_profile_begin / g4b_profile_end: one duration per call for its dominant kernel, -1 when that kernel is
+    masked out, results unchanged, misuse reported."""
+    import ctypes
+
+    from g4b_amd import _native
+
+    lib = _native.load()
+    B, H, G, D, W = 4, 8, 2, 256, 2048
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=61)
+    tds, ph = i32([W, 100, 1500, W + 9]), u8([2] * B)
+    ws = torch.empty(fa.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device="cuda")
+    fa.flash_attention(q, k, v, o, tds, ph, W, 2, scale=1 / 16, workspace=ws)
+    torch.cuda.synchronize()
+    expect = o.clone()
+    assert lib.g4b_profile_end(None, 0) == _native.G4B_ERR_INVALID_ARGUMENT
+    assert lib.g4b_profile_begin() == 0
+    assert lib.g4b_profile_begin() == _native.G4B_ERR_INVALID_ARGUMENT
+    o.zero_()
+    for mask in (0, 0, 2, 1):
+        fa.flash_attention(q, k, v, o, tds, ph, W, 2, scale=1 / 16, workspace=ws, kernel_mask=mask)
+    buf = (ctypes.c_float * 8)()
+    assert lib.g4b_profile_end(buf, 8) == 4
+    ts = list(buf[:4])
+    assert ts[2] == -1.0 and all(0 < t < 5.0 for t in (ts[0], ts[1], ts[3])), ts
+    torch.cuda.synchronize()
+    assert torch.equal(o, expect)
+    # a prefill-shaped call is timed the same way
+    q2, k2, v2, o2 = make_case(1, H, G, 256, D, 512, seed=62)
+    assert lib.g4b_profile_begin() == 0
+    fa.flash_attention(q2, k2, v2, o2, i32([512]), u8([1]), 512, 1, scale=1 / 16)
+    assert lib.g4b_profile_end(buf, 8) == 1 and 0 < buf[0] < 5.0
+
+
 def test_argument_errors_follow_the_reference(fa):
     B, H, G, D, W = 2, 8, 2, 256, 64
     q, k, v, o = make_case(B, H, G, 1, D, W, seed=10)

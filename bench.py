@@ -478,7 +478,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed steps first; the board needs some 20 ms of load before its clocks settle")
     ap.add_argument("--workload", default="decode_batched", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extra", action="store_true", help="time the primary workload only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -538,7 +539,7 @@ def main():
                 continue
             w = make(dev)
             steps = 3 if name == "mixed_step" else min(args.steps, 20)
-            r = measure(w, steps, min(args.warmup, 3))
+            r = measure(w, steps, 5 if name == "mixed_step" else min(args.warmup, 60))
             entry = {"ms_per_step": round(r["ms_per_step"], 4), "GB/s": round(r["GBps"], 1),
                      "TFLOP/s": round(r["TFLOPs"], 2), "roofline": r["roofline"]}
             if isinstance(w, MixedStep):

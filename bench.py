@@ -569,6 +569,8 @@ def main():
                    "detail": "fp16 Q/K/V ~ N(0,1) seeded, fp32 softmax accumulation"},
         "roofline": res["roofline"],
         "cpu_baseline": cpu,
+        "kernel_ms": {"avg": round(res["kernel_ms_avg"], 5), "median": round(res["kernel_ms_median"], 5),
+                      "event_pair_avg": round(res["event_pair_ms_avg"], 5), "launches": max(args.steps, 10)},
         "device": props.name,
         "extra": extra,
     }

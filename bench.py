@@ -89,11 +89,11 @@ class Workload:
         raise NotImplementedError
 
 
-def _randn_f16(shape, seed, device):
+def _randn_f16(shape, seed, device, dtype=None):
     import torch
 
     g = torch.Generator(device=device).manual_seed(seed)
-    return torch.randn(shape, generator=g, device=device, dtype=torch.float16)
+    return torch.randn(shape, generator=g, device=device, dtype=dtype or torch.float16)
 
 
 class BatchedDecode(Workload):
@@ -214,7 +214,7 @@ class Prefill(Workload):
 
     bound = "mfma"
 
-    def __init__(self, device, S, query_window=None, seed=0, dim=D):
+    def __init__(self, device, S, query_window=None, seed=0, dim=D, bf16=False):
         import torch
 
         from g4b_amd.kernels import fa2
@@ -225,9 +225,12 @@ class Prefill(Workload):
         D_ = self.D_ = dim
         if dim != D:
             self.name += f"_d{dim}"
-        self.q = _randn_f16((1, H, S, D_), seed + 1, device)
-        self.k = _randn_f16((1, G, S, D_), seed + 2, device)
-        self.v = _randn_f16((1, G, S, D_), seed + 3, device)
+        dt = torch.bfloat16 if bf16 else torch.float16
+        if bf16:
+            self.name += "_bf16"
+        self.q = _randn_f16((1, H, S, D_), seed + 1, device, dt)
+        self.k = _randn_f16((1, G, S, D_), seed + 2, device, dt)
+        self.v = _randn_f16((1, G, S, D_), seed + 3, device, dt)
         self.o = torch.empty_like(self.q)
         self.tds = torch.full((1,), S, dtype=torch.int32, device=device)
         self.phase = torch.full((1,), fa2.PHASE_PREFILL, dtype=torch.uint8, device=device)
@@ -387,6 +390,7 @@ WORKLOADS = {
     "prefill_causal_8192": lambda dev: Prefill(dev, 8192),
     "prefill_swa_8192": lambda dev: Prefill(dev, 8192, query_window=512),
     "prefill_causal_8192_d512": lambda dev: Prefill(dev, 8192, dim=512),
+    "prefill_causal_8192_bf16": lambda dev: Prefill(dev, 8192, bf16=True),
     "mixed_step": lambda dev: MixedStep(dev),
     "rope_append": lambda dev: RopeAppend(dev),
 }

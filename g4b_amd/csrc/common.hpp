@@ -56,7 +56,11 @@ struct BF16 {
         b2 v = {(__bf16)lo, (__bf16)hi};
         return __builtin_bit_cast(uint32_t, v);
     }
-    static G4B_DEV float sum2(uint32_t w, float acc) { return acc + lo(w) + hi(w); }
+    static G4B_DEV float sum2(uint32_t w, float acc) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        const b2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, w), ones, acc, false);
+    }
     static G4B_DEV float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
     static G4B_DEV float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 };

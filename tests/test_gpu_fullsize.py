@@ -121,6 +121,21 @@ def test_config3_prefill_8192(fa, qw):
     assert torch.equal(o3, o)
 
 
+def test_config3_prefill_8192_bf16(fa):
+    """Configuration 3b with bf16 q / caches / output (the other operand type of the same kernels)."""
+    from helpers import ATOL_BF16, RTOL_BF16
+
+    S = 8192
+    q, k, v = (randn16(shape, seed).bfloat16() for shape, seed in (((1, H, S, D), 1), ((1, G, S, D), 2), ((1, G, S, D), 3)))
+    o = torch.full_like(q, 777.0)
+    fa.flash_attention(q, k, v, o, i32([S]), u8([1]), S, 1, scale=SCALE)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    rows = [0, 1, 31, 32, 511, 512, 4095, 4096, 8190, 8191] + np.random.default_rng(5).integers(0, S, 10).tolist()
+    assert_close(got[0][:, rows], oracle_rows(q, k, v, 0, rows, S, S, S), atol=ATOL_BF16, rtol=RTOL_BF16, what="config 3b bf16")
+
+
 def test_config3_uniform_attention_is_the_running_mean(fa):
     """K = 0: every visible key has the same weight, so row i of a causal prefill is mean(V[0..i])."""
     S = 8192

@@ -1,0 +1,89 @@
+"""Seeded random sweep of small launches against the fp64 oracle: every combination the boundary accepts of head
+dimension, group size, query tokens, ring length, window, per-query window, stage, per-slot windows, dtypes, phases
+and lengths (empty slots, lengths below / at / beyond the window, wrapped rings), split and unsplit.  The fixed cases
+elsewhere follow the reference's shape list; this one looks for the corner nobody listed.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ATOL_BF16, RTOL_BF16, assert_close, i32, ix, oracle, u8
+
+pytestmark = pytest.mark.gpu
+
+N_CASES = 240
+
+
+def draw_case(rng):
+    D = int(rng.choice([128, 256, 512]))
+    R = int(rng.choice([1, 2, 4, 8, 16]))
+    G = int(rng.choice([1, 2, 3]))
+    H = R * G
+    Tq = int(rng.choice([1, 1, 2, 3, 5, 16, 33, 64, 100]))
+    kv_ctx = int(rng.integers(max(Tq, 8), 260))
+    W = int(rng.integers(max(Tq, 1), kv_ctx + 1))
+    B = int(rng.integers(1, 7))
+    phase_id = 2 if Tq == 1 and rng.random() < 0.7 else 1
+    phase = [phase_id if rng.random() < 0.75 else int(rng.choice([0, 3 - phase_id])) for _ in range(B)]
+    tds = []
+    for _ in range(B):
+        kind = rng.integers(0, 5)
+        if kind == 0:
+            tds.append(0 if Tq == 1 else Tq)  # nothing but the chunk itself (or an empty decode slot)
+        elif kind == 1:
+            tds.append(int(rng.integers(Tq, W + 1)))  # window not yet full
+        elif kind == 2:
+            tds.append(W)
+        else:
+            tds.append(int(rng.integers(W, 4 * kv_ctx)))  # ring wrapped
+    stage = ix.STAGE_FULL if rng.random() < 0.2 else ix.STAGE_CAUSAL
+    qwin = int(rng.integers(1, 2 * W)) if rng.random() < 0.3 else None
+    win = [int(rng.integers(Tq, W + 1)) for _ in range(B)] if rng.random() < 0.25 else None  # the caller keeps window >= Tq
+    bf16 = rng.random() < 0.25
+    q_f32 = rng.random() < 0.3
+    engine = rng.random() < 0.5
+    split = rng.random() < 0.5
+    scale = float(rng.choice([1.0, 1 / 16, 0.3]))
+    return dict(D=D, H=H, G=G, Tq=Tq, kv_ctx=kv_ctx, W=W, B=B, phase_id=phase_id, phase=phase, tds=tds, stage=stage, qwin=qwin,
+                win=win, bf16=bf16, q_f32=q_f32, engine=engine, split=split, scale=scale)
+
+
+@pytest.mark.parametrize("n", range(N_CASES))
+def test_random_launch(gpu_device, n):
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(1000 + n)
+    c = draw_case(rng)
+    print({k: v for k, v in c.items()}, flush=True)
+    B, H, G, Tq, D = c["B"], c["H"], c["G"], c["Tq"], c["D"]
+    cdt = torch.bfloat16 if c["bf16"] else torch.float16
+    qdt = torch.float32 if c["q_f32"] else cdt
+    gen = torch.Generator().manual_seed(2000 + n)
+    if c["engine"]:
+        q = torch.randn(B, Tq, H, D, generator=gen).to(qdt).cuda().permute(0, 2, 1, 3)
+        o = torch.full((B, Tq, H, D), 777.0, dtype=qdt, device="cuda").permute(0, 2, 1, 3)
+    else:
+        q = torch.randn(B, H, Tq, D, generator=gen).to(qdt).cuda()
+        o = torch.full((B, H, Tq, D), 777.0, dtype=qdt, device="cuda")
+    k = torch.randn(B, G, c["kv_ctx"], D, generator=gen).to(cdt).cuda()
+    v = torch.randn(B, G, c["kv_ctx"], D, generator=gen).to(cdt).cuda()
+    kw = dict(stage=c["stage"], scale=c["scale"], query_window=c["qwin"])
+    # the kernels feed the MFMA with q rounded to the cache's 16-bit type
+    ref = oracle(q.to(cdt), k, v, c["tds"], c["phase"], c["W"], c["phase_id"], window_sizes=c["win"], **kw)
+    if c["win"] is not None:
+        kw["window_sizes"] = i32(c["win"])
+    if c["split"]:
+        kw["workspace"] = torch.empty(max(fa2.workspace_bytes(B, H, G, Tq, D), 16), dtype=torch.uint8, device="cuda")
+    elif (H // G) * Tq > 16:
+        kw["workspace"] = False
+    fa2.flash_attention(q, k, v, o, i32(c["tds"]), u8(c["phase"]), c["W"], c["phase_id"], **kw)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if c["bf16"] else {}
+    sentinel = torch.tensor(777.0, dtype=qdt).float().item()  # 776 in bf16
+    for b in range(B):
+        if c["phase"][b] == c["phase_id"]:
+            assert_close(got[b], ref[b], what=f"case {n} slot {b}", **tol)
+        else:
+            assert (got[b] == sentinel).all(), f"case {n}: off-phase slot {b} was written"

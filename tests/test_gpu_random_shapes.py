@@ -87,3 +87,60 @@ def test_random_launch(gpu_device, n):
             assert_close(got[b], ref[b], what=f"case {n} slot {b}", **tol)
         else:
             assert (got[b] == sentinel).all(), f"case {n}: off-phase slot {b} was written"
+
+
+N_ROPE_CASES = 60
+
+
+@pytest.mark.parametrize("n", range(N_ROPE_CASES))
+def test_random_rope_append(gpu_device, n):
+    """RoPE + q/k RMSNorm + ring append in one launch against the oracle's composition: random head dimensions (the
+    value heads may differ), token counts up to the ring length, offsets that wrap, scratchpad layouts and dtypes,
+    cache dtypes, phase skip."""
+    from g4b_amd.kernels import rope
+    from oracle import rope_ref as rr
+
+    rng = np.random.default_rng(5000 + n)
+    D = int(rng.choice([64, 128, 256, 512]))
+    Dv = int(rng.choice([D, D, 128, 512]))
+    G = int(rng.choice([1, 2, 4]))
+    H = G * int(rng.choice([1, 2, 4, 8]))
+    B = int(rng.integers(1, 5))
+    T = int(rng.integers(1, 70))
+    t = int(rng.integers(1, T + 1))
+    offs = [int(rng.integers(0, 100000)) if rng.random() < 0.7 else int(rng.integers(0, T)) for _ in range(B)]
+    phase_id = int(rng.choice([1, 2]))
+    phase = [phase_id if rng.random() < 0.75 else 0 for _ in range(B)]
+    xdt = [torch.float32, torch.float32, torch.float16, torch.bfloat16][int(rng.integers(0, 4))]
+    cdt = torch.float16 if rng.random() < 0.6 else torch.bfloat16
+    engine = rng.random() < 0.6
+    print(dict(D=D, Dv=Dv, G=G, H=H, B=B, T=T, t=t, offs=offs, phase=phase, xdt=xdt, cdt=cdt, engine=engine), flush=True)
+    gen = torch.Generator().manual_seed(6000 + n)
+
+    def pad(heads, d):
+        if engine:
+            return torch.randn(B, t, heads, d, generator=gen).to(xdt).cuda().permute(0, 2, 1, 3)
+        return torch.randn(B, heads, t, d, generator=gen).to(xdt).cuda()
+
+    q, k, v = pad(H, D), pad(G, D), pad(G, Dv)
+    q_rsos, k_rsos, v_rsos = ((x.float() ** 2).sum(-1) for x in (q, k, v))
+    freqs = torch.from_numpy(rr.populate_rope_frequencies_ref(D // 2, 1e6).astype(np.float32)).cuda()
+    qw = (1 + 0.1 * torch.randn(D, generator=gen)).cuda()
+    kw = (1 + 0.1 * torch.randn(D, generator=gen)).cuda()
+    kc = torch.randn(B, G, T, D, generator=gen).to(cdt).cuda()
+    vc = torch.randn(B, G, T, Dv, generator=gen).to(cdt).cuda()
+    f = lambda x: x.float().cpu().numpy()  # noqa: E731
+    kc_ref, vc_ref = f(kc).copy(), f(vc).copy()
+    q_ref, _ = rr.rope_append_ref(f(q), f(k), f(v), f(freqs), np.array(offs), f(q_rsos), f(k_rsos), f(v_rsos), f(qw), f(kw), 1e-6,
+                                  kc_ref, vc_ref, np.array(phase), phase_id)
+    q0, k0 = q.clone(), k.clone()
+    rope.apply_rope_and_append(q, k, v, freqs, i32(offs), q_rsos, k_rsos, v_rsos, qw, kw, 1e-6, kc, vc, u8(phase), phase_id)
+    torch.cuda.synchronize()
+    x_tol = {torch.float32: 2e-4, torch.float16: 4e-3, torch.bfloat16: 3e-2}[xdt]
+    c_tol = 4e-3 if cdt == torch.float16 else 3e-2
+    # angles of up to 1e5 radians: the oracle's fp32 angle product is the reference, as in the kernel
+    np.testing.assert_allclose(f(q), q_ref, rtol=x_tol, atol=x_tol * 4)
+    np.testing.assert_allclose(f(kc), kc_ref, rtol=c_tol, atol=c_tol * 4)
+    np.testing.assert_allclose(f(vc), vc_ref, rtol=c_tol, atol=c_tol * 4)
+    assert torch.equal(k, k0)  # the K scratchpad is left alone
+    del q0

@@ -144,3 +144,39 @@ def test_random_rope_append(gpu_device, n):
     np.testing.assert_allclose(f(vc), vc_ref, rtol=c_tol, atol=c_tol * 4)
     assert torch.equal(k, k0)  # the K scratchpad is left alone
     del q0
+
+
+@pytest.mark.parametrize("n", range(40))
+def test_random_kv_append_is_bit_exact(gpu_device, n):
+    """Plain append (no normalisation): every ring row holds exactly the token the index formula puts there, in the
+    cache's dtype, and nothing else moved -- for random shapes, offsets (int32 or int64), phases and layouts."""
+    from g4b_amd.kernels.add_kv_to_cache import add_kv_to_cache
+
+    rng = np.random.default_rng(7000 + n)
+    D = 8 * int(rng.integers(1, 70))
+    G, B = int(rng.integers(1, 5)), int(rng.integers(1, 6))
+    T = int(rng.integers(1, 90))
+    t = int(rng.integers(1, T + 1))
+    offs = [int(rng.integers(0, 1 << 20)) for _ in range(B)]
+    use_phase = rng.random() < 0.6
+    phase = [1 if rng.random() < 0.7 else 2 for _ in range(B)]
+    xdt = [torch.float32, torch.float16, torch.bfloat16][int(rng.integers(0, 3))]
+    cdt = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
+    odt = torch.int64 if rng.random() < 0.5 else torch.int32
+    gen = torch.Generator().manual_seed(8000 + n)
+    if rng.random() < 0.5:
+        x = torch.randn(B, t, G, D, generator=gen).to(xdt).cuda().permute(0, 2, 1, 3)
+    else:
+        x = torch.randn(B, G, t, D, generator=gen).to(xdt).cuda()
+    cache0 = torch.randn(B, G, T, D, generator=gen).to(cdt).cuda()
+    cache = cache0.clone()
+    kw = dict(user_phase=u8(phase), phase=1) if use_phase else {}
+    add_kv_to_cache(x, cache, torch.tensor(offs, dtype=odt, device="cuda"), 1e-6, **kw)
+    torch.cuda.synchronize()
+    exp = cache0.clone()
+    for b in range(B):
+        if use_phase and phase[b] != 1:
+            continue
+        rows = (torch.arange(t) + offs[b]) % T
+        exp[b][:, rows.cuda(), :] = x[b].to(cdt)
+    assert torch.equal(cache, exp), dict(D=D, G=G, B=B, T=T, t=t, offs=offs, phase=phase if use_phase else None)

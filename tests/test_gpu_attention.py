@@ -285,7 +285,7 @@ def test_bound_plan_relaunches_with_new_device_data(fa):
 
 
 def test_one_shot_causal_prefill_2048(fa):
-    """BASELINE config 2: batch 1, seq 2048, 8 q heads / 2 kv heads, head dim 256, scale 1/16."""
+    """Benchmark configuration 2: batch 1, seq 2048, 8 q heads / 2 kv heads, head dim 256, scale 1/16."""
     B, H, G, Tq, D = 1, 8, 2, 2048, 256
     q, k, v, o = make_case(B, H, G, Tq, D, Tq, seed=0)
     ref = oracle(q, k, v, [Tq], [1], Tq, 1, scale=1 / 16)

@@ -1,4 +1,4 @@
-"""Parity at the full sizes of the benchmark configurations (BASELINE.json configs 1-5).
+"""Parity at the full sizes of the five benchmark configurations.
 
 The fp64 oracle is evaluated on sampled slots / query rows so that it finishes in seconds; in
 addition, size-independent properties are checked on the whole output: split and unsplit launches

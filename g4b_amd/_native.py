@@ -14,7 +14,7 @@ G4B_ERR_WORKSPACE = -3
 G4B_ERR_LAUNCH = -4
 
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class AttnArgs(C.Structure):
@@ -50,6 +50,7 @@ class AttnArgs(C.Structure):
         ("query_window", C.c_int32),
         ("num_workers", C.c_int32),
         ("kernel_mask", C.c_int32),
+        ("use_fp32_dot", C.c_int32),
         ("scale", C.c_float),
     ]
 

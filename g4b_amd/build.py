@@ -27,7 +27,8 @@ SOURCES = ["api.hip", "attn_decode.hip", "attn_prefill.hip", "attn_prefill_wide.
 
 # packed-fp32 VALU forms are kept off: the compiler must not form v_pk_{add,mul,fma}_f32
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-variable", "-Wno-unknown-pragmas"]
+COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fno-honor-nans", f"--offload-arch={ARCH}", "-Wall", "-Wno-unused-variable", "-Wno-unknown-pragmas",
+                "-Wno-inline-asm"]  # the M0 clobber of dma_set_base is deliberate
 
 
 def hipcc() -> str:
@@ -105,6 +106,17 @@ def check_wait_discipline() -> dict:
                     ins = l.strip()
                     if foreign.search(ins) and not ins.startswith(allowed):
                         raise RuntimeError(f"{m.group(1)}: `{ins}` inside the hand-counted wait region")
+                # M0 carries the LDS destination of the direct loads from one dma_set_base (`s_mov_b32 m0` + `s_nop 0`,
+                # one asm block) to the loads that follow it: any other write to M0 in the kernel would misplace a tile.
+                code = [l.strip() for l in body if l.strip() and not l.strip().startswith((";", ".", "//"))]
+                for j, ins in enumerate(code):
+                    ops = ins.split(None, 1)
+                    writes_m0 = len(ops) == 2 and ops[0].startswith(("s_", "v_readlane", "v_readfirstlane")) and \
+                        re.match(r"m0\b", ops[1]) is not None
+                    if writes_m0 and not (ops[0] == "s_mov_b32" and j + 1 < len(code) and code[j + 1].startswith("s_nop 0")):
+                        raise RuntimeError(f"{m.group(1)}: `{ins}` writes M0 outside dma_set_base")
+                    if ops[0].startswith(("s_movrel", "v_movrel")):
+                        raise RuntimeError(f"{m.group(1)}: `{ins}` uses M0 as an index next to the direct loads")
                 seen[m.group(1)] = len(mfma)
                 i = end
     return seen

@@ -192,6 +192,9 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     p.qwin = a->query_window;
     p.c = a->scale * 1.44269504088896340736f;
     p.kernel_mask = (a->kernel_mask & 3) ? (a->kernel_mask & 3) : 3;
+    // a query wider than the cache type: f32 over f16 / bf16, f16 over bf16
+    const bool q_wider = a->q_dtype == G4B_DT_F32 || (a->q_dtype == G4B_DT_F16 && a->kv_dtype == G4B_DT_BF16);
+    p.q_split = (a->use_fp32_dot && q_wider) ? 1 : 0;
 
     const int64_t rows = (int64_t)p.R * p.Tq;
     hipError_t e;
@@ -212,7 +215,8 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
-        const int bm = prefill_rows_per_workgroup(a->D);
+        // a split query halves the rows of a head-dimension-512 workgroup
+        const int bm = prefill_rows_per_workgroup(a->D) / ((a->D == 512 && p.q_split) ? 2 : 1);
         if (bm % p.R)
             return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide %d for prefill-shaped launches with head_dim %d", p.R, bm, a->D);
         p.split_slots = 0;

@@ -52,7 +52,10 @@ G4B_DEV float pick(const f4& c, int e, int cls) {
 //
 // lds_part != nullptr: the un-normalised result goes to that LDS block ([16 rows][D] floats, then [16 rows][2] of
 // (reference, sum)) whatever the segment covers; the caller merges the blocks of its waves.
-template <int D, int CL, class T, int DH>
+//
+// QS: the query is wider than the cache type and enters the first product as two operands (rounded value, rounding
+// error), so the scores see the unrounded query.
+template <int D, int CL, class T, int DH, bool QS>
 G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb, float* xch,
                             float* lds_part = nullptr) {
     constexpr int DL = D / DH;         // columns this wave owns
@@ -90,6 +93,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
     row_range(p, si, 0, dummy, hi_min);
 
     u4 qf[NC];
+    u4 qf_lo[QS ? NC : 1];
     {
         const int64_t qoff =
             (int64_t)bb * p.q_s[0] + (int64_t)(g * p.R + hh) * p.q_s[1] + (int64_t)ti * p.q_s[2] + hv * DL;
@@ -97,7 +101,13 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
         for (int c = 0; c < NC; ++c) {
             const int piece = cls + CL * g4 + 4 * CL * c;
             u4 z = {0, 0, 0, 0};
-            qf[c] = row_ok ? load8_as<T>(p.q, qoff + piece * 8, p.q_dt) : z;
+            if constexpr (QS) {
+                qf[c] = z;
+                qf_lo[c] = z;
+                if (row_ok) load8_split<T>(p.q, qoff + piece * 8, p.q_dt, qf[c], qf_lo[c]);
+            } else {
+                qf[c] = row_ok ? load8_as<T>(p.q, qoff + piece * 8, p.q_dt) : z;
+            }
         }
     }
 
@@ -146,7 +156,10 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
         for (int tau = 0; tau < NT; ++tau) {
             f4 c4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < NC; ++c) c4 = T::mfma16(kreg[tau][c], qf[c], c4);
+            for (int c = 0; c < NC; ++c) {
+                if constexpr (QS) c4 = T::mfma16(kreg[tau][c], qf_lo[c], c4);
+                c4 = T::mfma16(kreg[tau][c], qf[c], c4);
+            }
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 float x = pick<CL>(c4, e, cls);
@@ -253,7 +266,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
     }
 }
 
-template <int D, int CL, class T, int DH>
+template <int D, int CL, class T, int DH, bool QS>
 __global__ __launch_bounds__(64 * DH, 1) void attn_decode_worker(const AttnParams p) {
     __shared__ float xch_buf[DH > 1 ? 2 * DH * 8 * 64 : 1];
     float* xch = xch_buf;
@@ -265,7 +278,7 @@ __global__ __launch_bounds__(64 * DH, 1) void attn_decode_worker(const AttnParam
         // no workspace: worker w owns the whole pair w
         const int bb = w / G, g = w % G;
         const int tlb = slot_tiles(p, bb);
-        if (tlb > 0) decode_segment<D, CL, T, DH>(p, w, bb, g, 0, tlb, tlb, xch);
+        if (tlb > 0) decode_segment<D, CL, T, DH, QS>(p, w, bb, g, 0, tlb, tlb, xch);
         return;
     }
 
@@ -300,7 +313,7 @@ __global__ __launch_bounds__(64 * DH, 1) void attn_decode_worker(const AttnParam
                 const int64_t fs = (int64_t)ex + (int64_t)g * tlb;
                 const int t0 = (int)(max(ws, fs) - fs);
                 const int t1 = (int)(min(we, fs + tlb) - fs);
-                if (t1 > t0) decode_segment<D, CL, T, DH>(p, w, bb, g, t0, t1, tlb, xch);
+                if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, w, bb, g, t0, t1, tlb, xch);
             }
         }
         carry += __shfl(incl, 63);
@@ -315,7 +328,7 @@ constexpr int DEC_PAIR_WAVES = 4;
 template <int D>
 constexpr int dec_pair_smem() { return DEC_PAIR_WAVES * (16 * D + 32) * (int)sizeof(float); }
 
-template <int D, int CL, class T>
+template <int D, int CL, class T, bool QS>
 __global__ __launch_bounds__(64 * DEC_PAIR_WAVES, 1) void attn_decode_pair(const AttnParams p) {
     extern __shared__ __align__(16) float pair_smem[];
     constexpr int BLK = 16 * D + 32;  // floats per wave block
@@ -329,7 +342,7 @@ __global__ __launch_bounds__(64 * DEC_PAIR_WAVES, 1) void attn_decode_pair(const
     float* mine = pair_smem + wave * BLK;
     const int t0 = wave * tl / DEC_PAIR_WAVES, t1 = (wave + 1) * tl / DEC_PAIR_WAVES;
     if (t1 > t0) {
-        decode_segment<D, CL, T, 1>(p, 0, bb, g, t0, t1, tl, nullptr, mine);
+        decode_segment<D, CL, T, 1, QS>(p, 0, bb, g, t0, t1, tl, nullptr, mine);
     } else if ((tid & 63) < 16) {
         mine[16 * D + (tid & 63) * 2] = -INFINITY;  // this wave brought no keys
         mine[16 * D + (tid & 63) * 2 + 1] = 0.f;
@@ -470,22 +483,22 @@ static bool decode_pair_path(const AttnParams& p, int D) {
     return D <= 256 && p.win_arr == nullptr && (p.W < p.KV_CTX ? p.W : p.KV_CTX) <= DEC_PAIR_MAX_KEYS;
 }
 
-template <int D, int CL, class T>
+template <int D, int CL, class T, bool QS>
 static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
     if constexpr (D <= 256) {
         if (decode_pair_path(p, D)) {
             static uint64_t attr_done = 0;
-            hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_decode_pair<D, CL, T>), dec_pair_smem<D>(), attr_done);
+            hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_decode_pair<D, CL, T, QS>), dec_pair_smem<D>(), attr_done);
             if (e != hipSuccess) return e;
             if (p.kernel_mask & 1)
-                G4B_LAUNCH_DOMINANT((attn_decode_pair<D, CL, T>), dim3(p.B * p.G), dim3(64 * DEC_PAIR_WAVES), dec_pair_smem<D>(),
+                G4B_LAUNCH_DOMINANT((attn_decode_pair<D, CL, T, QS>), dim3(p.B * p.G), dim3(64 * DEC_PAIR_WAVES), dec_pair_smem<D>(),
                                     stream, p);
             return hipGetLastError();
         }
     }
     constexpr int DH = D > 256 ? D / 256 : 1;  // waves per worker: each owns at most 256 columns
     if (p.kernel_mask & 1) {
-        G4B_LAUNCH_DOMINANT((attn_decode_worker<D, CL, T, DH>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64 * DH), 0, stream,
+        G4B_LAUNCH_DOMINANT((attn_decode_worker<D, CL, T, DH, QS>), dim3(p.NW > 0 ? p.NW : p.B * p.G), dim3(64 * DH), 0, stream,
                             p);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -497,9 +510,14 @@ static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
 template <int D, class T>
 static hipError_t launch_decode_cl(const AttnParams& p, hipStream_t stream) {
     const int rows = p.R * p.Tq;
-    if (rows <= 4) return launch_decode_t<D, 4, T>(p, stream);
-    if (rows <= 8) return launch_decode_t<D, 2, T>(p, stream);
-    return launch_decode_t<D, 1, T>(p, stream);
+    if (p.q_split) {
+        if (rows <= 4) return launch_decode_t<D, 4, T, true>(p, stream);
+        if (rows <= 8) return launch_decode_t<D, 2, T, true>(p, stream);
+        return launch_decode_t<D, 1, T, true>(p, stream);
+    }
+    if (rows <= 4) return launch_decode_t<D, 4, T, false>(p, stream);
+    if (rows <= 8) return launch_decode_t<D, 2, T, false>(p, stream);
+    return launch_decode_t<D, 1, T, false>(p, stream);
 }
 
 hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream) {

@@ -42,7 +42,9 @@ struct PfSmem {
     static constexpr int VSWZ = (D >= 256) ? 7 : 3;  // (V row & VSWZ) selects the 64-byte group swizzle
 };
 
-template <int D, class T>
+// QS: the query is wider than the cache type (fp32 scratchpads over a 16-bit cache) and enters S^T = K Q^T as two
+// B operands, the rounded value and its rounding error, against the same K fragments.
+template <int D, class T, bool QS>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     using SM = PfSmem<D>;
     extern __shared__ __align__(16) char smem[];
@@ -240,10 +242,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
         stage_whole_tile(kt0, true, 0);
         // Q as B operand: lane (row n32, half h2), step c: d = 16c + 8*h2 .. +8 (loaded behind the staging loads)
         u4 qf[KSTEPS];
+        u4 qf_lo[QS ? KSTEPS : 1];
 #pragma unroll
         for (int c = 0; c < KSTEPS; ++c) {
             u4 z = {0, 0, 0, 0};
-            qf[c] = row_ok ? load8_as<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt) : z;
+            if constexpr (QS) {
+                qf[c] = z;
+                qf_lo[c] = z;
+                if (row_ok) load8_split<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt, qf[c], qf_lo[c]);
+            } else {
+                qf[c] = row_ok ? load8_as<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt) : z;
+            }
         }
         vm_wait_all();
         __syncthreads();
@@ -266,6 +275,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                 if (idx + PF_PD < QK_STEPS) {
                     abuf[idx % PF_PD] = k_issue(idx + PF_PD);
                     abuf[(idx + 1) % PF_PD] = k_issue(idx + 1 + PF_PD);
+                }
+                if constexpr (QS) {
+                    s_cur[0] = T::mfma32(a0, qf_lo[idx >> 1], s_cur[0]);
+                    s_cur[1] = T::mfma32(a1, qf_lo[idx >> 1], s_cur[1]);
                 }
                 s_cur[0] = T::mfma32(a0, qf[idx >> 1], s_cur[0]);
                 s_cur[1] = T::mfma32(a1, qf[idx >> 1], s_cur[1]);
@@ -322,6 +335,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
                 if (idx + PF_PD < QK_STEPS) {
                     abuf[idx % PF_PD] = k_issue(idx + PF_PD);
                     abuf[(idx + 1) % PF_PD] = k_issue(idx + 1 + PF_PD);
+                }
+                if constexpr (QS) {
+                    s_nxt[0] = T::mfma32(a0, qf_lo[idx >> 1], s_nxt[0]);
+                    s_nxt[1] = T::mfma32(a1, qf_lo[idx >> 1], s_nxt[1]);
                 }
                 s_nxt[0] = T::mfma32(a0, qf[idx >> 1], s_nxt[0]);
                 s_nxt[1] = T::mfma32(a1, qf[idx >> 1], s_nxt[1]);
@@ -463,7 +480,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     }
 }
 
-template <int D, class T>
+template <int D, class T, bool QS>
 static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     const int TOKB = PF_BM / p.R;
     const int slots = p.part_o ? p.split_slots : 1;
@@ -471,9 +488,9 @@ static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
     dim3 grid(blocks);
     const int smem = 4 * PfSmem<D>::TILE;
     static uint64_t attr_done = 0;
-    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T>), smem, attr_done);
+    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T, QS>), smem, attr_done);
     if (e != hipSuccess) return e;
-    if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_kernel<D, T>), grid, dim3(256), smem, stream, p);
+    if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_kernel<D, T, QS>), grid, dim3(256), smem, stream, p);
     if (slots > 1 && (p.kernel_mask & 2)) {
         const int items = min(p.B, slots / 2);  // more active slots than this are never split
         hipLaunchKernelGGL((attn_prefill_combine<D>), dim3(items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS)), dim3(256), 0, stream, p);
@@ -482,12 +499,20 @@ static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
 }
 
 hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_t stream) {
-    if (kv_dt == DT_F16) {
-        if (D == 256) return launch_prefill_t<256, F16>(p, stream);
-        if (D == 128) return launch_prefill_t<128, F16>(p, stream);
+    if (p.q_split) {
+        if (kv_dt == DT_F16) {
+            if (D == 256) return launch_prefill_t<256, F16, true>(p, stream);
+            if (D == 128) return launch_prefill_t<128, F16, true>(p, stream);
+        } else {
+            if (D == 256) return launch_prefill_t<256, BF16, true>(p, stream);
+            if (D == 128) return launch_prefill_t<128, BF16, true>(p, stream);
+        }
+    } else if (kv_dt == DT_F16) {
+        if (D == 256) return launch_prefill_t<256, F16, false>(p, stream);
+        if (D == 128) return launch_prefill_t<128, F16, false>(p, stream);
     } else {
-        if (D == 256) return launch_prefill_t<256, BF16>(p, stream);
-        if (D == 128) return launch_prefill_t<128, BF16>(p, stream);
+        if (D == 256) return launch_prefill_t<256, BF16, false>(p, stream);
+        if (D == 128) return launch_prefill_t<128, BF16, false>(p, stream);
     }
     return hipErrorInvalidValue;
 }

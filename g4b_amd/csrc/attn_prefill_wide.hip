@@ -12,6 +12,12 @@
 // operand, V read with ds_read_b64_tr_b16, v_mfma_f32_32x32x16, P kept in registers, exp2 softmax in fp32 with lazy
 // rescaling.  The next tile's loads are issued one per two MFMA steps of the first product and waited for at the
 // barrier that closes the tile.
+//
+// QS (a query wider than the cache type, to enter K Q^T unrounded): there is no register left for a second Q block,
+// so a wave owns 16 rows and the 32 columns of its B operand hold their rounded values (columns 0..15) and their
+// rounding errors (columns 16..31).  The two halves of S^T are added across the lane pair (n, n + 16) right after the
+// first product, which leaves both lanes with the score of the unrounded query; from there on the lanes of a pair
+// carry the same row (the second product computes it twice) and a workgroup covers 64 rows.
 #include "common.hpp"
 #include "launch.hpp"
 #include "prefill_combine.hpp"
@@ -21,13 +27,22 @@ namespace g4b {
 
 constexpr int PW_D = 512;                // head dimension
 constexpr int PW_BN = 32;                // keys per tile
-constexpr int PW_BM = PF_BM;             // query rows per workgroup
+constexpr int PW_BM = PF_BM;             // query rows per workgroup (half of it for a split query)
 constexpr int PW_ROW = PW_D * 2;         // bytes per K or V row
 constexpr int PW_TILE = PW_BN * PW_ROW;  // bytes per staged tile
 constexpr int PW_SMEM = 4 * PW_TILE;
 constexpr int PW_PD = 4;                 // LDS operand fetches in flight
 
-template <class T>
+// Sum over the lane pair (l, l ^ 16): v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even
+// rows of its second, leaving (row 0, row 0, row 2, row 2) and (row 1, row 1, row 3, row 3).
+G4B_DEV float row16_pair_sum(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    const u2 r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+template <class T, bool QS>
 __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams p) {
     extern __shared__ __align__(16) char smem[];
     constexpr int D = PW_D, ROW = PW_ROW, TILE = PW_TILE;
@@ -41,7 +56,9 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
     const int lane = tid & 63, wave = tid >> 6;
     const int n32 = lane & 31, h2 = lane >> 5;
     const int R = p.R, Tq = p.Tq, KV_CTX = p.KV_CTX;
-    const int TOKB = PW_BM / R;
+    constexpr int WROWS = QS ? 16 : 32;  // query rows per wave
+    constexpr int BM = 4 * WROWS;
+    const int TOKB = BM / R;
     __shared__ int sh_scan[8];
     int n_active;
     nth_active_slot(p, -1, n_active, sh_scan);
@@ -64,7 +81,7 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
     row_range(p, si, tok_last, lo_max, hi_wg);
 
     // this lane's row
-    const int rrow = wave * 32 + n32;
+    const int rrow = wave * WROWS + (QS ? (n32 & 15) : n32);
     const int hh = rrow / TOKB;
     const int ti = tok0 + rrow % TOKB;
     const bool row_ok = ti < Tq;
@@ -188,7 +205,13 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
 #pragma unroll
             for (int c = 0; c < KSTEPS; ++c) {
                 u4 z = {0, 0, 0, 0};
-                qf[c] = row_ok ? load8_as<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt) : z;
+                if constexpr (QS) {
+                    u4 qh = z, ql = z;
+                    if (row_ok) load8_split<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt, qh, ql);
+                    qf[c] = (n32 < 16) ? qh : ql;
+                } else {
+                    qf[c] = row_ok ? load8_as<T>(p.q, qoff + c * 16 + h2 * 8, p.q_dt) : z;
+                }
             }
             vm_wait_all();
             __syncthreads();
@@ -224,6 +247,11 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
                         if (idx / 2 < CHUNKS) dma_chunk(idx / 2, tk, false, kdst);
                         else dma_chunk(idx / 2 - CHUNKS, tv, true, vdst);
                     }
+                }
+
+                if constexpr (QS) {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) s[j] = row16_pair_sum(s[j]);  // K q_hi + K q_lo
                 }
 
                 // ---- edge tiles: mask
@@ -313,12 +341,12 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
     const bool partial = nsplit > 1;
     const float inv = partial ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);
     char* wbase = smem + wave * (32 * 256 * 4);
-    if (partial && h2 == 0 && row_ok) {
+    if (partial && h2 == 0 && row_ok && (!QS || n32 < 16)) {
         const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hh)) * Tq + ti;
         p.part_ml[prow * 2] = (m_run == -INFINITY) ? 0.f : m_run;
         p.part_ml[prow * 2 + 1] = l_tot;
     }
-    const int tokb_shift = __ffs(TOKB) - 1;  // TOKB = 128 / R is a power of two
+    const int tokb_shift = __ffs(TOKB) - 1;  // TOKB = BM / R is a power of two
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -331,9 +359,9 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
                 *reinterpret_cast<f4*>(wbase + n32 * 1024 + ((pc ^ (n32 & 15)) * 16)) = v;
             }
 #pragma unroll 4
-        for (int row = 0; row < 32; ++row) {
+        for (int row = 0; row < WROWS; ++row) {  // with a split query the LDS rows 16..31 are copies of 0..15
             const int pc = lane;  // 64 lanes x 16 bytes = 256 fp32 columns of one row
-            const int rr = wave * 32 + row;
+            const int rr = wave * WROWS + row;
             const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
             const f4 v = *reinterpret_cast<const f4*>(wbase + row * 1024 + ((pc ^ (row & 15)) * 16));
             if (tr < Tq) {
@@ -349,14 +377,14 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
     }
 }
 
-template <class T>
+template <class T, bool QS>
 static hipError_t launch_prefill_wide_t(const AttnParams& p, hipStream_t stream) {
     const int slots = p.part_o ? p.split_slots : 1;
-    const int blocks = prefill_grid(p, PW_BM);
+    const int blocks = prefill_grid(p, QS ? PW_BM / 2 : PW_BM);
     static uint64_t attr_done = 0;
-    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<T>), PW_SMEM, attr_done);
+    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<T, QS>), PW_SMEM, attr_done);
     if (e != hipSuccess) return e;
-    if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_wide_kernel<T>), dim3(blocks), dim3(256), PW_SMEM, stream, p);
+    if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_wide_kernel<T, QS>), dim3(blocks), dim3(256), PW_SMEM, stream, p);
     if (slots > 1 && (p.kernel_mask & 2)) {
         const int items = min(p.B, slots / 2);  // more active slots than this are never split
         hipLaunchKernelGGL((attn_prefill_combine<PW_D>), dim3(items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS)), dim3(256), 0,
@@ -366,7 +394,8 @@ static hipError_t launch_prefill_wide_t(const AttnParams& p, hipStream_t stream)
 }
 
 hipError_t launch_attn_prefill_wide(const AttnParams& p, int kv_dt, hipStream_t stream) {
-    return kv_dt == DT_F16 ? launch_prefill_wide_t<F16>(p, stream) : launch_prefill_wide_t<BF16>(p, stream);
+    if (p.q_split) return kv_dt == DT_F16 ? launch_prefill_wide_t<F16, true>(p, stream) : launch_prefill_wide_t<BF16, true>(p, stream);
+    return kv_dt == DT_F16 ? launch_prefill_wide_t<F16, false>(p, stream) : launch_prefill_wide_t<BF16, false>(p, stream);
 }
 
 }  // namespace g4b

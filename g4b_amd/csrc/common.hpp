@@ -96,6 +96,37 @@ G4B_DEV u4 load8_as(const void* base, int64_t elem_off, int dt) {
     return r;
 }
 
+// The same eight elements as a pair of operands hi + lo: hi is the value rounded to T, lo the rounding error rounded
+// to T again, so that K.hi + K.lo reproduces the product with the unrounded query to about twice T's mantissa.  For a
+// source type that T holds exactly lo is zero.
+template <class T>
+G4B_DEV void load8_split(const void* base, int64_t elem_off, int dt, u4& hi, u4& lo) {
+    float x[8];
+    if (dt == DT_F32) {
+        const f4* p = reinterpret_cast<const f4*>(static_cast<const float*>(base) + elem_off);
+        const f4 a = p[0], b = p[1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[i] = a[i];
+            x[4 + i] = b[i];
+        }
+    } else {
+        const u4 raw = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = raw[i];
+            x[2 * i] = (dt == DT_F16) ? F16::lo(w) : BF16::lo(w);
+            x[2 * i + 1] = (dt == DT_F16) ? F16::hi(w) : BF16::hi(w);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t h = T::pack2(x[2 * i], x[2 * i + 1]);
+        hi[i] = h;
+        lo[i] = T::pack2(x[2 * i] - T::lo(h), x[2 * i + 1] - T::hi(h));
+    }
+}
+
 // Store eight consecutive output elements (dtype chosen at run time) from eight floats.
 G4B_DEV void store8(void* base, int64_t elem_off, int dt, const float (&v)[8]) {
     if (dt == DT_F32) {
@@ -235,6 +266,7 @@ struct AttnParams {
     int32_t NW;  // number of decode workers (waves) the key tiles are dealt to
     int32_t split_slots;  // prefill: (active slot, key split) pairs the partial buffers hold; <= 1 = never split
     int32_t kernel_mask;  // bit 0: main kernel, bit 1: merge kernel
+    int32_t q_split;      // 1: a query wider than the cache type enters K Q^T as a hi + lo pair of operands
     float c;     // softmax scale * log2(e)
 };
 

@@ -70,7 +70,8 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     const int rows = 256 / tpr;          // tokens per workgroup
     const int tt = blockIdx.x * rows + threadIdx.x / tpr;
     const int j0 = (threadIdx.x % tpr) * 8;
-    if (tt >= p.t) return;
+    // threads beyond rows * tpr (D / 16 does not divide 256) would alias the next workgroup's first token
+    if ((int)threadIdx.x >= rows * tpr || tt >= p.t) return;
 
     const int32_t off = p.offsets[(int64_t)b * p.off_s];
     const float pos = (float)(off + tt);  // rope.py:180: integer position, converted once

@@ -145,6 +145,7 @@ def _bind(
         raise ValueError("query_window must be a positive int or None")
     a.num_workers = int(num_workers)
     a.kernel_mask = int(kernel_mask)
+    a.use_fp32_dot = 1 if use_fp32_dot else 0
     a.scale = float(scale)
 
     ws = None if workspace is False else workspace
@@ -205,9 +206,13 @@ def flash_attention(
       split keys across workgroups, as in the reference; the partials themselves live in a
       private workspace (or ``workspace=``) with this library's own layout, and the contents of
       ``partial_*`` are left unspecified.
-    * ``use_grouped_query_tile``, ``warp_specialize``, ``is_hopper``, ``use_fp32_dot``: tuning
-      knobs of the Triton kernel; accepted and ignored (the GQA group is always packed and the
-      products always run on fp16/bf16 MFMA with fp32 accumulation).
+    * ``use_grouped_query_tile``, ``warp_specialize``, ``is_hopper``: tuning knobs of the Triton
+      kernel; accepted and ignored (the GQA group is always packed).
+    * ``use_fp32_dot`` (``fa2.py:85-88``): ``False`` rounds a wider query to the cache's 16-bit type
+      before ``K Q^T``, as the reference's ``q.to(tl.float16)`` does; ``True`` (what the engine passes
+      with its fp32 scratchpads, ``g4b/models/gemma4e.py:606``) feeds the product with the query as
+      the sum of two 16-bit operands, value and rounding error, so the scores are those of the
+      unrounded query.  The products run on fp16/bf16 MFMA with fp32 accumulation either way.
     * ``stage``: ``STAGE_CAUSAL`` or ``STAGE_FULL``.
 
     Keyword-only extensions, with defaults that reproduce the reference:

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define G4B_ATTN_ABI_VERSION 1
+#define G4B_ATTN_ABI_VERSION 2
 
 enum g4b_status {
     G4B_OK = 0,
@@ -71,6 +71,12 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *                 wave, or a pair of waves when D = 512.  Ignored by
  *                 prefill-shaped launches, which choose their key split from the number of in-phase
  *                 slots on the device.
+ *   use_fp32_dot  the reference's USE_FP32_DOT (fa2.py:85-88,126-129): 0 = the query is rounded to the cache's 16-bit
+ *                 type before K Q^T, as the reference's `q.to(tl.float16)` does; non-zero = a query of a wider type
+ *                 (f32 over any cache, f16 over a bf16 cache) enters K Q^T as the sum of two 16-bit operands, its
+ *                 rounded value and its rounding error, so the scores are those of the unrounded query.  The engine
+ *                 passes fp32 q with use_fp32_dot=True and scale 1.0 (g4b/models/gemma4e.py:30,606).  No effect when
+ *                 q already has the cache's type.
  *   kernel_mask   profiling aid.  0 = run every kernel of the launch.  Otherwise bit 0 selects the
  *                 main attention kernel and bit 1 the split-merge kernel, so that each can be timed
  *                 on its own; results are only complete with both.
@@ -105,6 +111,7 @@ typedef struct g4b_attn_args {
     int32_t query_window;
     int32_t num_workers;
     int32_t kernel_mask;
+    int32_t use_fp32_dot;
     float scale;
 } g4b_attn_args;
 

@@ -49,6 +49,9 @@ CASES = [
     ("chunk_d256", 2, 8, 2, 96, 256, [0, 16384]),
     ("chunk_ragged_d128", 3, 4, 4, 37, 128, [5, 999, 20000]),
     ("chunk_d64", 1, 2, 1, 300, 64, [123]),
+    # D / 16 does not divide the 256 threads of a workgroup: the spare threads must stay out of the next block's token
+    ("chunk_d96", 2, 4, 2, 130, 96, [7, 3000]),
+    ("chunk_d160", 1, 4, 1, 77, 160, [41]),
 ]
 
 

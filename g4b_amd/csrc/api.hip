@@ -5,14 +5,43 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 #include <utility>
 #include <vector>
 
 #include "launch.hpp"
 
+// Scratch of g4b_attn_forward_static_scratch: split partials of one launch.  Every device the library runs on holds
+// its own copy of this array at its own address until the process ends; host code reaches it only through the
+// per-device pointer that static_scratch_ptr() obtains with hipGetSymbolAddress.
+constexpr size_t kStaticScratchBytes = (size_t)G4B_ATTN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 thread_local char g_err[512] = "";
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+hipError_t static_scratch_ptr(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!ptr) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return hipSuccess;
+}
 
 // g4b_profile_begin .. g4b_profile_end: one (start, stop) event pair per timed call of this thread
 thread_local bool g_profiling = false;
@@ -237,6 +266,34 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     profile_disarm();
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
     return G4B_OK;
+}
+
+int g4b_static_scratch_init(void) {
+    void* ptr = nullptr;
+    const hipError_t e = static_scratch_ptr(&ptr);
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "static scratch: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
+uint64_t g4b_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int g4b_attn_forward_static_scratch(const g4b_attn_args* a, void* stream) {
+    if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
+    if (a->workspace) return fail(G4B_ERR_INVALID_ARGUMENT, "g4b_attn_forward_static_scratch brings its own scratch: workspace must be NULL");
+    const uint64_t need = g4b_attn_workspace_bytes(a->B, a->H, a->G, a->Tq, a->D, a->num_workers);
+    if (need > kStaticScratchBytes)
+        return fail(G4B_ERR_WORKSPACE, "this launch splits keys through %llu bytes of partials, the static scratch holds %llu; "
+                    "use g4b_attn_forward with a workspace of that size",
+                    (unsigned long long)need, (unsigned long long)kStaticScratchBytes);
+    g4b_attn_args b = *a;
+    if (need) {
+        void* ptr = nullptr;
+        const hipError_t e = static_scratch_ptr(&ptr);
+        if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "static scratch: %s", hipGetErrorString(e));
+        b.workspace = ptr;
+        b.workspace_bytes = kStaticScratchBytes;
+    }
+    return g4b_attn_forward(&b, stream);
 }
 
 int g4b_kv_append(const g4b_kv_append_args* a, void* stream) {

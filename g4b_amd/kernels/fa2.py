@@ -148,9 +148,17 @@ def _bind(
     a.use_fp32_dot = 1 if use_fp32_dot else 0
     a.scale = float(scale)
 
-    ws = None if workspace is False else workspace
+    static = isinstance(workspace, str)
+    if static and workspace != "static":
+        raise ValueError('workspace must be a uint8 tensor, None, False or "static"')
+    ws = None if (workspace is False or static) else workspace
     if workspace is False:
         pass  # no scratch at all: nothing is split
+    elif static:
+        # the library's own scratch array (g4b_attn_forward_static_scratch): nothing is allocated here or there; a
+        # decode launch still splits only when the reference's split buffers were passed
+        if (H // G) * Tq <= MAX_DECODE_ROWS and max_kv_splits <= 1:
+            static = False
     elif ws is None and (H // G) * Tq <= MAX_DECODE_ROWS:
         if max_kv_splits > 1:
             ws = _private_workspace(q, workspace_bytes(B, H, G, Tq, D, num_workers))
@@ -164,7 +172,8 @@ def _bind(
         a.workspace = ws.data_ptr()
         a.workspace_bytes = int(ws.numel()) * int(ws.element_size()) if hasattr(ws, "numel") else int(ws.nbytes)
 
-    return a, (q, k_cache, v_cache, o, time_dim_sizes, user_phase, window_sizes, ws)
+    entry = lib.g4b_attn_forward_static_scratch if static else lib.g4b_attn_forward
+    return a, (q, k_cache, v_cache, o, time_dim_sizes, user_phase, window_sizes, ws), entry
 
 
 def flash_attention(
@@ -220,20 +229,22 @@ def flash_attention(
     * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
       ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
       ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
-      used for split partials instead of the private one; ``False`` = use none and never split); ``num_workers``; ``kernel_mask`` (profiling:
+      used for split partials instead of the private one; ``False`` = use none and never split; ``"static"`` = the
+      library's built-in scratch array through ``g4b_attn_forward_static_scratch``, which allocates nothing and
+      refuses launches whose partials exceed ``g4b_static_scratch_bytes()``; calls that overlap on one GPU must not
+      share it); ``num_workers``; ``kernel_mask`` (profiling:
       bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
 
     Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
     ignore (``g4b/models/gemma4e.py:593-607``).
     """
-    a, _keep = _bind(
+    a, _keep, entry = _bind(
         q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, partial_o, partial_l, partial_m,
         use_grouped_query_tile=use_grouped_query_tile, warp_specialize=warp_specialize, is_hopper=is_hopper,
         use_fp32_dot=use_fp32_dot, stage=stage, scale=scale, query_window=query_window, window_sizes=window_sizes,
         workspace=workspace, num_workers=num_workers, kernel_mask=kernel_mask,
     )
-    lib = _native.load()
-    _native.check(lib.g4b_attn_forward(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    _native.check(entry(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
     return None, None
 
 
@@ -246,13 +257,12 @@ class AttentionPlan:
     plan holds references to the tensors it points into.
     """
 
-    def __init__(self, args, keep):
-        self._args, self._keep = args, keep
-        self._lib = _native.load()
+    def __init__(self, args, keep, entry):
+        self._args, self._keep, self._entry = args, keep, entry
         self._ref = C.byref(args)
 
     def launch(self, stream=None) -> None:
-        rc = self._lib.g4b_attn_forward(self._ref, C.c_void_p(U.current_stream() if stream is None else int(stream)))
+        rc = self._entry(self._ref, C.c_void_p(U.current_stream() if stream is None else int(stream)))
         if rc:
             _native.check(rc)
 
@@ -260,5 +270,5 @@ class AttentionPlan:
 def plan_flash_attention(*args, **kwargs) -> AttentionPlan:
     """Same arguments as :func:`flash_attention` (without ``stream``); returns an :class:`AttentionPlan`."""
     kwargs.pop("stream", None)
-    a, keep = _bind(*args, **kwargs)
-    return AttentionPlan(a, keep)
+    a, keep, entry = _bind(*args, **kwargs)
+    return AttentionPlan(a, keep, entry)

@@ -129,6 +129,27 @@ uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, i
 int32_t g4b_attn_default_workers(void);
 
 /*
+ * g4b_attn_forward_static_scratch: g4b_attn_forward for callers that cannot allocate.  It has no counterpart in the
+ * reference; it is for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc, which
+ * have no place to get the split-KV workspace from.  Same arguments and results as g4b_attn_forward with a workspace
+ * of g4b_attn_workspace_bytes(...) bytes, except that `workspace` must be NULL: the split partials go to an array of
+ * G4B_ATTN_STATIC_SCRATCH_BYTES bytes that is part of the library's device image (one copy per GPU the library runs
+ * on, held until the process ends).  The call itself allocates and frees nothing.  A launch whose partials need more
+ * than that is refused with G4B_ERR_WORKSPACE (the limit covers every prefill shape up to head dimension 512 and
+ * decode batches of about a thousand (slot, kv head) pairs at the default worker count).  No kernel reads scratch
+ * that the same call has not written, so nothing is cleared between calls; all calls on one GPU share the array, so
+ * calls that overlap on one GPU (two streams, two threads) race -- serialise them or give one of them a workspace.
+ *
+ * g4b_static_scratch_init looks the array's device address up for the current device (the first
+ * g4b_attn_forward_static_scratch on a device does the same); call it once per device at load when the first launch
+ * would otherwise happen under stream capture.
+ */
+#define G4B_ATTN_STATIC_SCRATCH_BYTES (68u << 20)
+int g4b_attn_forward_static_scratch(const g4b_attn_args* args, void* stream);
+int g4b_static_scratch_init(void);
+uint64_t g4b_static_scratch_bytes(void);
+
+/*
  * g4b_kv_append replaces add_kv_to_cache() (g4b/kernels/add_kv_to_cache.py:84-186):
  *   cache[b, g, (t + cache_offsets[b]) % T, :] = x[b, g, t, :] * (x_rsos ? rsqrt(x_rsos[b,g,t] / D + eps) : 1)
  * for slots with user_phase[b] == phase (all slots when user_phase is NULL).

@@ -1,0 +1,91 @@
+"""g4b_attn_forward_static_scratch (split partials in the library's own device array, no allocation) against
+g4b_attn_forward with a caller-provided workspace: same kernels, same partition, so the outputs must be bit-identical.
+
+Two calls in a row per shape family, the second with a smaller input, so that the second call runs over what the
+first left in the scratch array.  pytest collects this file last (its name sorts after every other test file), so a failure here hides no other test.
+"""
+
+import ctypes as C
+
+import pytest
+import torch
+
+from helpers import i32, ix, make_case, partials, u8
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fa(gpu_device):
+    from g4b_amd.kernels import fa2
+
+    return fa2
+
+
+def run_both(fa, q, k, v, tds, phase, W, phase_id, parts, **kw):
+    """-> (output with an explicit workspace, output through the static scratch), both via the C ABI."""
+    B, H, Tq, D = q.shape
+    G = k.shape[1]
+    need = fa.workspace_bytes(B, H, G, Tq, D)
+    assert need > 0, "the shape must be one that splits keys"
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    o_ws = torch.full_like(q, 777.0)
+    fa.flash_attention(q, k, v, o_ws, tds, phase, W, phase_id, *parts, workspace=ws, **kw)
+    o_st = torch.full_like(q, 777.0)
+    fa.flash_attention(q, k, v, o_st, tds, phase, W, phase_id, *parts, workspace="static", **kw)
+    torch.cuda.synchronize()
+    return o_ws, o_st
+
+
+def test_decode_split_two_calls_second_smaller(fa):
+    from g4b_amd import _native
+
+    lib = _native.load()
+    assert lib.g4b_static_scratch_init() == 0, _native.last_error()
+    assert lib.g4b_static_scratch_bytes() == 68 << 20
+    for B, D, W, seed in ((24, 256, 6000, 1), (5, 256, 1500, 2), (6, 512, 3000, 3), (2, 512, 700, 4)):
+        print(f"static scratch decode B={B} D={D} W={W}", flush=True)
+        H, G = 8, 2
+        q, k, v, _ = make_case(B, H, G, 1, D, W, seed=seed)
+        tds = [W if b % 2 == 0 else max(1, W // (b + 1)) for b in range(B)]
+        phase = [ix.PHASE_DECODE if b % 5 != 4 else ix.PHASE_PREFILL for b in range(B)]
+        o_ws, o_st = run_both(fa, q, k, v, i32(tds), u8(phase), W, ix.PHASE_DECODE, partials(16, B, H, 1, D), scale=0.0625)
+        assert torch.equal(o_ws, o_st), f"B={B} D={D}: static scratch differs from the workspace path"
+        for b in range(B):
+            if phase[b] != ix.PHASE_DECODE:
+                assert (o_st[b] == 777.0).all()
+            else:
+                assert (o_st[b] != 777.0).any()
+
+
+def test_prefill_chunk_split_two_calls_second_smaller(fa):
+    for Tq, D, ctx, seed in ((256, 256, 3000, 5), (96, 256, 700, 6), (128, 512, 1500, 7), (64, 512, 300, 8)):
+        print(f"static scratch chunk Tq={Tq} D={D} ctx={ctx}", flush=True)
+        B, H, G = 3, 8, 2
+        kv_ctx = ctx + Tq + 64
+        q, k, v, _ = make_case(B, H, G, Tq, D, kv_ctx, seed=seed)
+        tds = [ctx + Tq, 0, Tq]
+        phase = [ix.PHASE_PREFILL, ix.PHASE_DECODE, ix.PHASE_PREFILL]
+        o_ws, o_st = run_both(fa, q, k, v, i32(tds), u8(phase), kv_ctx, ix.PHASE_PREFILL, (), scale=0.0625)
+        assert torch.equal(o_ws, o_st), f"Tq={Tq} D={D}: static scratch differs from the workspace path"
+        assert (o_st[1] == 777.0).all() and (o_st[0] != 777.0).any()
+
+
+def test_rejects_what_does_not_fit_and_a_foreign_workspace(fa):
+    from g4b_amd import _native
+
+    lib = _native.load()
+    B, H, G, D, W = 2, 8, 2, 256, 512
+    q, k, v, o = make_case(B, H, G, 1, D, W, seed=9)
+    args, keep, entry = fa._bind(q, k, v, o, i32([W, W]), u8([2, 2]), W, 2, *partials(4, B, H, 1, D), workspace="static",
+                                 num_workers=1 << 20)
+    assert entry is lib.g4b_attn_forward_static_scratch or entry == lib.g4b_attn_forward_static_scratch
+    rc = lib.g4b_attn_forward_static_scratch(C.byref(args), None)
+    assert rc == _native.G4B_ERR_WORKSPACE, rc
+    assert "static scratch holds" in _native.last_error()
+    args.num_workers = 0
+    args.workspace = q.data_ptr()
+    args.workspace_bytes = 1 << 30
+    rc = lib.g4b_attn_forward_static_scratch(C.byref(args), None)
+    assert rc == _native.G4B_ERR_INVALID_ARGUMENT, rc
+    torch.cuda.synchronize()

@@ -146,6 +146,8 @@ EXPORTS = {
     "g4b_attn_forward_static_scratch": (C.c_int, [C.POINTER(AttnArgs), C.c_void_p]),
     "g4b_static_scratch_init": (C.c_int, []),
     "g4b_static_scratch_bytes": (C.c_uint64, []),
+    "g4b_attn_forward_mixed": (C.c_int, [C.POINTER(AttnArgs), C.POINTER(AttnArgs), C.c_void_p]),
+    "g4b_attn_mixed_workspace_bytes": (C.c_uint64, [C.c_int32] * 10),
     "g4b_attn_workspace_bytes": (C.c_uint64, [C.c_int32] * 6),
     "g4b_attn_default_workers": (C.c_int32, []),
     "g4b_kv_append": (C.c_int, [C.POINTER(KvAppendArgs), C.c_void_p]),

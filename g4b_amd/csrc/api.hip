@@ -10,6 +10,8 @@
 #include <vector>
 
 #include "launch.hpp"
+#include "prefill_combine.hpp"
+#include "prefill_map.hpp"
 
 // Scratch of g4b_attn_forward_static_scratch: split partials of one launch.  Every device the library runs on holds
 // its own copy of this array at its own address until the process ends; host code reaches it only through the
@@ -153,7 +155,9 @@ uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, i
     return decode_slots(B, G, nw) * (uint64_t)rows * (uint64_t)(D + 2) * sizeof(float);
 }
 
-int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
+// Host-side validation of one argument block and its translation into kernel parameters (everything except the
+// workspace, which depends on the kind of launch).
+static int fill_attn_params(const g4b_attn_args* a, g4b::AttnParams& p) {
     if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
     if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->time_dim_sizes || !a->user_phase)
         return fail(G4B_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, time_dim_sizes and user_phase must be non-NULL");
@@ -190,7 +194,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         return fail(G4B_ERR_UNSUPPORTED, "KV_CTX * D * 2 bytes must be below 2 GiB per (slot, kv head)");
     if (a->num_workers < 0 || a->num_workers > (1 << 20)) return fail(G4B_ERR_INVALID_ARGUMENT, "num_workers out of range");
 
-    g4b::AttnParams p{};
+    p = g4b::AttnParams{};
     p.q = a->q;
     p.k = a->k_cache;
     p.v = a->v_cache;
@@ -224,7 +228,12 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     // a query wider than the cache type: f32 over f16 / bf16, f16 over bf16
     const bool q_wider = a->q_dtype == G4B_DT_F32 || (a->q_dtype == G4B_DT_F16 && a->kv_dtype == G4B_DT_BF16);
     p.q_split = (a->use_fp32_dot && q_wider) ? 1 : 0;
+    return G4B_OK;
+}
 
+int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
+    g4b::AttnParams p;
+    if (const int rc = fill_attn_params(a, p)) return rc;
     const int64_t rows = (int64_t)p.R * p.Tq;
     hipError_t e;
     if (rows <= kMaxDecodeRows) {
@@ -265,6 +274,105 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     }
     profile_disarm();
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "attention launch failed: %s", hipGetErrorString(e));
+    return G4B_OK;
+}
+
+// ---- one launch for a mixed step ----------------------------------------------------------------------------------
+// The chip's 256 compute units are shared out between the two halves on the host, from static shapes only: the decode
+// half gets what lets its stream run at full rate, the chunk the rest.
+namespace {
+constexpr int kMixedCus = 256;
+constexpr int kMixedDecodeBlocks = 80;  // decode workgroups (four one-wave workers each) asked for by default
+
+struct MixedShape {
+    int split_slots;     // (active slot, key split) pairs of the prefill half; <= 1 = unsplit
+    g4b::MixedPlan plan;
+    int nw;              // decode workers (0 with the pair path or without a workspace)
+    uint64_t pf_bytes, dec_bytes;
+};
+
+// B, H, G, D, KV_CTX, W, window_sizes are shared; tq_pf / tq_dec are the query tokens per slot of the two halves.
+MixedShape mixed_shape(int B, int H, int G, int D, int tq_pf, int tq_dec, bool pair_path, int num_workers, bool with_ws) {
+    MixedShape m{};
+    const int R = H / G, tokb = 128 / R;
+    const int per_slot = ((tq_pf + tokb - 1) / tokb) * G;  // prefill workgroups one slot brings unsplit
+    int nd = pair_path ? B * G : (num_workers > 0 ? (num_workers + 3) / 4 : kMixedDecodeBlocks);
+    if (!with_ws && !pair_path) nd = (B * G + 3) / 4;  // one worker per pair
+    int slots = with_ws ? (kMixedCus - nd) / per_slot : 1;
+    slots = slots < 1 ? 1 : (slots > kPrefillMaxSplitSlots ? kPrefillMaxSplitSlots : slots);
+    if (!pair_path && with_ws && num_workers <= 0 && slots * per_slot + nd < kMixedCus) nd = kMixedCus - slots * per_slot;
+    m.split_slots = slots >= 2 ? slots : 0;
+    m.nw = (pair_path || !with_ws) ? 0 : nd * 4;
+    m.plan.nd_blocks = nd;
+    m.plan.pair_path = pair_path ? 1 : 0;
+    m.pf_bytes = (uint64_t)m.split_slots * H * tq_pf * (uint64_t)(D + 2) * sizeof(float);
+    m.dec_bytes = m.nw ? decode_slots(B, G, m.nw) * (uint64_t)R * tq_dec * (uint64_t)(D + 2) * sizeof(float) : 0;
+    return m;
+}
+}  // namespace
+
+uint64_t g4b_attn_mixed_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq_prefill, int32_t Tq_decode, int32_t D,
+                                        int32_t KV_CTX, int32_t ctx_window_size, int32_t has_window_sizes, int32_t num_workers) {
+    if (B < 1 || H < 1 || G < 1 || Tq_prefill < 1 || Tq_decode < 1 || D < 1 || H % G || 128 % (H / G)) return 0;
+    const int W = ctx_window_size < KV_CTX ? ctx_window_size : KV_CTX;
+    const bool pair = D <= 256 && !has_window_sizes && W <= g4b::DEC_PAIR_MAX_KEYS;
+    const MixedShape m = mixed_shape(B, H, G, D, Tq_prefill, Tq_decode, pair, num_workers, true);
+    return ((m.pf_bytes + 255) & ~(uint64_t)255) + m.dec_bytes;
+}
+
+int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* decode, void* stream) {
+    g4b::AttnParams pp, pd;
+    if (const int rc = fill_attn_params(prefill, pp)) return rc;
+    if (const int rc = fill_attn_params(decode, pd)) return rc;
+    const g4b_attn_args *a = prefill, *d = decode;
+    if (a->k_cache != d->k_cache || a->v_cache != d->v_cache || a->time_dim_sizes != d->time_dim_sizes ||
+        a->user_phase != d->user_phase || a->window_sizes != d->window_sizes || a->B != d->B || a->H != d->H || a->G != d->G ||
+        a->D != d->D || a->KV_CTX != d->KV_CTX || a->kv_dtype != d->kv_dtype || a->ctx_window_size != d->ctx_window_size ||
+        a->k_stride_b != d->k_stride_b || a->v_stride_b != d->v_stride_b || a->time_dim_sizes_stride != d->time_dim_sizes_stride ||
+        a->user_phase_stride != d->user_phase_stride || a->window_sizes_stride != d->window_sizes_stride)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "the two halves of a mixed launch must share the caches, the per-slot arrays, "
+                    "B, H, G, D, KV_CTX, the cache dtype and ctx_window_size");
+    if (a->phase == d->phase) return fail(G4B_ERR_INVALID_ARGUMENT, "the two halves of a mixed launch serve different phases");
+    if ((int64_t)pp.R * pp.Tq <= kMaxDecodeRows || (int64_t)pd.R * pd.Tq > kMaxDecodeRows)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "mixed launch: the first block must be prefill-shaped ((H/G)*Tq > %d), the second "
+                    "decode-shaped", kMaxDecodeRows);
+    if (a->D != 256) return fail(G4B_ERR_UNSUPPORTED, "mixed launch is built for head_dim 256 (got %d)", a->D);
+    if (128 % pp.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide 128 for prefill-shaped launches", pp.R);
+    if (pp.q_split != pd.q_split)
+        return fail(G4B_ERR_UNSUPPORTED, "mixed launch: both halves must take the same query precision path (same q dtype and use_fp32_dot)");
+    if (a->kernel_mask != d->kernel_mask) return fail(G4B_ERR_INVALID_ARGUMENT, "mixed launch: kernel_mask must agree");
+
+    const bool pair = g4b::decode_pair_path(pd, a->D);
+    const bool with_ws = a->workspace != nullptr;
+    const MixedShape m = mixed_shape(a->B, a->H, a->G, a->D, a->Tq, d->Tq, pair, d->num_workers, with_ws);
+    if (with_ws) {
+        // one workspace, passed with the prefill block: the chunk's partials first, the decode partials after them
+        const uint64_t pf_span = (m.pf_bytes + 255) & ~(uint64_t)255;
+        if (a->workspace_bytes < pf_span + m.dec_bytes)
+            return fail(G4B_ERR_WORKSPACE, "workspace holds %llu bytes, %llu needed for this mixed launch",
+                        (unsigned long long)a->workspace_bytes, (unsigned long long)(pf_span + m.dec_bytes));
+        if (!aligned16(a->workspace)) return fail(G4B_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+        if (m.split_slots) {
+            pp.split_slots = m.split_slots;
+            pp.part_o = static_cast<float*>(a->workspace);
+            pp.part_ml = pp.part_o + (uint64_t)m.split_slots * a->H * a->Tq * a->D;
+        }
+        if (m.nw) {
+            pd.NW = m.nw;
+            pd.part_o = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + pf_span);
+            pd.part_ml = pd.part_o + decode_slots(a->B, a->G, m.nw) * (uint64_t)pd.R * pd.Tq * (uint64_t)a->D;
+        }
+    }
+    g4b::MixedPlan mp = m.plan;
+    mp.npx = (g4b::prefill_grid(pp) + 7) / 8;
+    mp.combine_pf = g4b::prefill_combine_grid(pp);
+    mp.combine_dec = pair ? 0 : a->B * a->G * pd.R * pd.Tq;
+    if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
+    const hipError_t e = a->kv_dtype == G4B_DT_F16
+                             ? g4b::launch_attn_mixed_f16(pp, pd, mp, a->D, static_cast<hipStream_t>(stream))
+                             : g4b::launch_attn_mixed_bf16(pp, pd, mp, a->D, static_cast<hipStream_t>(stream));
+    profile_disarm();
+    if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "mixed attention launch failed: %s", hipGetErrorString(e));
     return G4B_OK;
 }
 

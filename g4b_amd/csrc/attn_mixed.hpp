@@ -1,0 +1,80 @@
+// One launch for a mixed step: the prefill-phase slots (a chunk of query tokens each) and the decode-phase slots
+// (one query token each) of the same batch, over the same caches.
+//
+// The two halves want different things from the chip.  The chunk is bound by the matrix pipes and scales with the
+// number of compute units it gets; the decode stream is bound by HBM and reaches its full rate with a wave on about
+// a third of the SIMDs (384 single-wave workers read as fast as 1024).  Launched one after the other, each half
+// leaves the other's resource idle.  Here one grid carries both: workgroup ids are dealt so that every XCD gets the
+// same mix, `npx` prefill workgroups per XCD first and the decode workgroups after them; a prefill workgroup runs the
+// body of the prefill kernel, a decode workgroup is four single-wave workers of the streaming kernel (or one
+// (slot, kv head) pair of the short-window variant).  Both kinds occupy a compute unit alone (registers, LDS), so
+// the hardware places prefill and decode workgroups side by side on different units and the chunk's matrix work runs
+// under the stream's memory time.  A second launch merges the split partials of both halves.
+#pragma once
+#include "attn_decode.hpp"
+#include "attn_prefill.hpp"
+#include "launch.hpp"
+
+namespace g4b {
+
+template <int D, int CL, class T, bool QS>
+__global__ __launch_bounds__(256) void attn_mixed_kernel(const AttnParams pp, const AttnParams pd, const MixedPlan mp) {
+    extern __shared__ __align__(16) char smem[];
+    __shared__ int sh_scan[8];
+    const int x = blockIdx.x & 7, j = blockIdx.x >> 3;  // workgroups go to the XCDs round-robin by id
+    if (j < mp.npx) {
+        prefill_body<D, T, QS>(pp, j * 8 + x, smem, sh_scan);
+        return;
+    }
+    const int d = (j - mp.npx) * 8 + x;
+    if (d >= mp.nd_blocks) return;
+    if (mp.pair_path) {
+        decode_pair_body<D, CL, T, QS>(pd, d, reinterpret_cast<float*>(smem));
+    } else {
+        decode_worker_body<D, CL, T, 1, QS>(pd, d * 4 + (int)(threadIdx.x >> 6), nullptr);
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_mixed_combine(const AttnParams pp, const AttnParams pd, const MixedPlan mp) {
+    __shared__ int sh_scan[8];
+    __shared__ DecodeCombineSmem<D> sm;
+    if ((int)blockIdx.x < mp.combine_pf) {
+        prefill_combine_body<D>(pp, blockIdx.x, sh_scan);
+        return;
+    }
+    const int d = blockIdx.x - mp.combine_pf, rows = pd.R * pd.Tq;
+    decode_combine_body<D>(pd, d / rows, d % rows, sm);
+}
+
+template <int D, int CL, class T, bool QS>
+static hipError_t launch_mixed_t(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream) {
+    constexpr int smem_pf = 4 * PfSmem<D>::TILE, smem_pair = dec_pair_smem<D>();
+    constexpr int smem = smem_pf > smem_pair ? smem_pf : smem_pair;
+    static uint64_t attr_done = 0;
+    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_mixed_kernel<D, CL, T, QS>), smem, attr_done);
+    if (e != hipSuccess) return e;
+    const int grid = 8 * (mp.npx + (mp.nd_blocks + 7) / 8);
+    if (pp.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_mixed_kernel<D, CL, T, QS>), dim3(grid), dim3(256), smem, stream, pp, pd, mp);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if ((pp.kernel_mask & 2) && mp.combine_pf + mp.combine_dec > 0)
+        hipLaunchKernelGGL((attn_mixed_combine<D>), dim3(mp.combine_pf + mp.combine_dec), dim3(256), 0, stream, pp, pd, mp);
+    return hipGetLastError();
+}
+
+template <class T>
+static hipError_t launch_mixed_dtype(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, int D, hipStream_t stream) {
+    const int rows = pd.R * pd.Tq;
+    if (D != 256) return hipErrorInvalidValue;
+    if (pp.q_split) {
+        if (rows <= 4) return launch_mixed_t<256, 4, T, true>(pp, pd, mp, stream);
+        if (rows <= 8) return launch_mixed_t<256, 2, T, true>(pp, pd, mp, stream);
+        return launch_mixed_t<256, 1, T, true>(pp, pd, mp, stream);
+    }
+    if (rows <= 4) return launch_mixed_t<256, 4, T, false>(pp, pd, mp, stream);
+    if (rows <= 8) return launch_mixed_t<256, 2, T, false>(pp, pd, mp, stream);
+    return launch_mixed_t<256, 1, T, false>(pp, pd, mp, stream);
+}
+
+}  // namespace g4b

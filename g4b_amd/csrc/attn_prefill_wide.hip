@@ -385,11 +385,8 @@ static hipError_t launch_prefill_wide_t(const AttnParams& p, hipStream_t stream)
     hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<T, QS>), PW_SMEM, attr_done);
     if (e != hipSuccess) return e;
     if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_wide_kernel<T, QS>), dim3(blocks), dim3(256), PW_SMEM, stream, p);
-    if (slots > 1 && (p.kernel_mask & 2)) {
-        const int items = min(p.B, slots / 2);  // more active slots than this are never split
-        hipLaunchKernelGGL((attn_prefill_combine<PW_D>), dim3(items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS)), dim3(256), 0,
-                           stream, p);
-    }
+    if (slots > 1 && (p.kernel_mask & 2))
+        hipLaunchKernelGGL((attn_prefill_combine<PW_D>), dim3(prefill_combine_grid(p)), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -38,12 +38,32 @@ inline hipError_t allow_dynamic_smem(const void* kernel, int bytes, uint64_t& do
     return e;
 }
 
+// Decode-shaped launches, host-side choice (static in the launch arguments, so a recorded graph keeps it): the
+// one-kernel variant (a workgroup of four waves per (slot, kv head) pair, merged through LDS) when no slot can bring
+// more than DEC_PAIR_MAX_KEYS keys (four tiles per wave; beyond that the waves' sequential tiles cost more than the
+// second launch saves).
+constexpr int DEC_PAIR_MAX_KEYS = 512;
+inline bool decode_pair_path(const AttnParams& p, int D) {
+    return D <= 256 && p.win_arr == nullptr && (p.W < p.KV_CTX ? p.W : p.KV_CTX) <= DEC_PAIR_MAX_KEYS;
+}
+
 // rows = (H/G) * Tq <= 16, D in {128, 256, 512}; kv_dt in {DT_F16, DT_BF16}
 hipError_t launch_attn_decode(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
 // any Tq; (H/G) must divide 128; D in {128, 256}
 hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_t stream);
 // any Tq; (H/G) must divide 128; D = 512
 hipError_t launch_attn_prefill_wide(const AttnParams& p, int kv_dt, hipStream_t stream);
+
+// One launch for the prefill-phase slots (pp: rows > 16) and the decode-phase slots (pd: rows <= 16) of a batch.
+struct MixedPlan {
+    int npx;          // prefill workgroups per XCD (grid slots; the prefill body drops the surplus)
+    int nd_blocks;    // decode workgroups
+    int pair_path;    // 1: short-window decode, one workgroup per (slot, kv head) pair
+    int combine_pf;   // merge workgroups of the prefill half
+    int combine_dec;  // merge workgroups of the decode half
+};
+hipError_t launch_attn_mixed_f16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, int D, hipStream_t stream);
+hipError_t launch_attn_mixed_bf16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, int D, hipStream_t stream);
 
 struct KvAppendParams {
     const void* x;

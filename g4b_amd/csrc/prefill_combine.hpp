@@ -45,10 +45,9 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
-    __shared__ int sh_scan[8];
+G4B_DEV void prefill_combine_body(const AttnParams& p, const int bid, int* sh_scan) {
     const int tblocks = (p.Tq + PFC_ROWS - 1) / PFC_ROWS;
-    const int a_idx = blockIdx.x / (p.H * tblocks), h = (blockIdx.x / tblocks) % p.H, tb = blockIdx.x % tblocks;
+    const int a_idx = bid / (p.H * tblocks), h = (bid / tblocks) % p.H, tb = bid % tblocks;
     int n_active;
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);
     const int nsplit = prefill_splits(p.split_slots, n_active);
@@ -57,6 +56,20 @@ __global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) 
     else if (nsplit <= 4) prefill_combine_rows<D, 4>(p, a_idx, b, h, tb, nsplit);
     else if (nsplit <= 8) prefill_combine_rows<D, 8>(p, a_idx, b, h, tb, nsplit);
     else prefill_combine_rows<D, 16>(p, a_idx, b, h, tb, nsplit);
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
+    __shared__ int sh_scan[8];
+    prefill_combine_body<D>(p, blockIdx.x, sh_scan);
+}
+
+// Workgroups the merge kernel of a split prefill-shaped launch needs (0 = the launch never splits).
+inline int prefill_combine_grid(const AttnParams& p) {
+    const int slots = p.part_o ? p.split_slots : 1;
+    if (slots <= 1) return 0;
+    const int items = p.B < slots / 2 ? p.B : slots / 2;  // more active slots than this are never split
+    return items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS);
 }
 
 }  // namespace g4b

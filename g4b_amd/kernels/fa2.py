@@ -27,8 +27,6 @@ PHASE_DECODE = 2
 
 MAX_DECODE_ROWS = 16  # (H/G) * Tq up to which a launch takes the split-KV streaming kernel
 
-_private_workspaces: dict = {}
-
 
 def workspace_bytes(B: int, H: int, G: int, Tq: int, D: int, num_workers: int = 0) -> int:
     """Bytes of scratch that let a launch of this shape split keys: over ``num_workers`` waves when it is
@@ -36,23 +34,36 @@ def workspace_bytes(B: int, H: int, G: int, Tq: int, D: int, num_workers: int = 
     return int(_native.load().g4b_attn_workspace_bytes(B, H, G, Tq, D, num_workers))
 
 
-def _private_workspace(q, nbytes: int):
-    """Per-device scratch owned by this module, created on first use and grown on demand.
+def mixed_workspace_bytes(B: int, H: int, G: int, Tq_prefill: int, Tq_decode: int, D: int, KV_CTX: int, ctx_window_size: int,
+                          has_window_sizes: bool = False, num_workers: int = 0) -> int:
+    """Bytes of scratch that let both halves of a mixed launch (``decode_q=`` / ``decode_o=``) split keys."""
+    return int(_native.load().g4b_attn_mixed_workspace_bytes(B, H, G, Tq_prefill, Tq_decode, D, KV_CTX, ctx_window_size,
+                                                             1 if has_window_sizes else 0, num_workers))
 
-    The reference sizes its split buffers once at load (``g4b/models/gemma4e.py:819-821``) and
-    compiles its kernels during warm-up; this allocation likewise happens on the first call with a
-    given shape, i.e. before a graph is recorded.  Callers that must not allocate at all pass
-    ``workspace=`` explicitly.
-    """
-    import torch
 
-    dev = q.device if hasattr(q, "device") else torch.device("cuda", torch.cuda.current_device())
-    key = str(dev)
-    ws = _private_workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-        _private_workspaces[key] = ws
-    return ws
+def _bind_mixed(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, decode_q, decode_o, decode_phase,
+                workspace, **kw):
+    """Argument blocks of the two halves of a mixed launch and the call that launches them as one grid."""
+    if decode_q is None or decode_o is None:
+        raise ValueError("decode_q and decode_o go together")
+    if isinstance(workspace, str):
+        raise ValueError("a mixed launch takes workspace=<uint8 tensor> (see mixed_workspace_bytes) or none")
+    kw = dict(kw)
+    num_workers = kw.pop("num_workers", 0)
+    a, keep_a, _ = _bind(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, workspace=False, **kw)
+    d, keep_d, _ = _bind(decode_q, k_cache, v_cache, decode_o, time_dim_sizes, user_phase, ctx_window_size, decode_phase,
+                         workspace=False, num_workers=num_workers, **kw)
+    ws = None if workspace is False else workspace
+    if ws is not None:
+        a.workspace = ws.data_ptr()
+        a.workspace_bytes = int(ws.numel()) * int(ws.element_size())
+    lib = _native.load()
+    d_ref = C.byref(d)
+
+    def entry(a_ref, stream):
+        return lib.g4b_attn_forward_mixed(a_ref, d_ref, stream)
+
+    return a, (keep_a, keep_d, d, ws), entry
 
 
 def _bind(
@@ -148,26 +159,24 @@ def _bind(
     a.use_fp32_dot = 1 if use_fp32_dot else 0
     a.scale = float(scale)
 
-    static = isinstance(workspace, str)
-    if static and workspace != "static":
+    if isinstance(workspace, str) and workspace != "static":
         raise ValueError('workspace must be a uint8 tensor, None, False or "static"')
-    ws = None if (workspace is False or static) else workspace
+    static = False
+    ws = None
     if workspace is False:
         pass  # no scratch at all: nothing is split
-    elif static:
-        # the library's own scratch array (g4b_attn_forward_static_scratch): nothing is allocated here or there; a
-        # decode launch still splits only when the reference's split buffers were passed
-        if (H // G) * Tq <= MAX_DECODE_ROWS and max_kv_splits <= 1:
-            static = False
-    elif ws is None and (H // G) * Tq <= MAX_DECODE_ROWS:
-        if max_kv_splits > 1:
-            ws = _private_workspace(q, workspace_bytes(B, H, G, Tq, D, num_workers))
-    elif ws is None:
-        # prefill-shaped: shapes whose in-phase slots may bring fewer workgroups than the chip has CUs
-        # (chunked prefill, short prompts) split every item's keys and merge; other shapes need none
-        need = workspace_bytes(B, H, G, Tq, D, 0)
-        if need:
-            ws = _private_workspace(q, need)
+    elif workspace is None or isinstance(workspace, str):
+        # Nothing is ever allocated here: the split partials go to the library's own scratch array
+        # (g4b_attn_forward_static_scratch).  A decode-shaped launch splits only when the reference's split buffers
+        # were passed (fa2.py:658); a prefill shape whose in-phase slots may bring fewer workgroups than the chip has
+        # compute units (chunked prefill, short prompts) splits every item's keys.  A launch whose partials would not
+        # fit the array runs unsplit.
+        decode_shaped = (H // G) * Tq <= MAX_DECODE_ROWS
+        need = workspace_bytes(B, H, G, Tq, D, num_workers if decode_shaped else 0)
+        wanted = need > 0 and (max_kv_splits > 1 if decode_shaped else True)
+        static = wanted and need <= int(lib.g4b_static_scratch_bytes())
+    else:
+        ws = workspace
     if ws is not None:
         a.workspace = ws.data_ptr()
         a.workspace_bytes = int(ws.numel()) * int(ws.element_size()) if hasattr(ws, "numel") else int(ws.nbytes)
@@ -201,6 +210,9 @@ def flash_attention(
     num_workers: int = 0,
     kernel_mask: int = 0,
     stream=None,
+    decode_q=None,
+    decode_o=None,
+    decode_phase: int = PHASE_DECODE,
 ):
     """``o[b, h, i] = softmax(scale * q[b, h, i] . K_b^T + mask) V_b`` for every in-phase slot ``b``.
 
@@ -212,9 +224,9 @@ def flash_attention(
       rows of ``o`` stay untouched.
     * ``partial_o/l/m``: the reference's split-KV scratch.  All three or none
       (``ValueError`` otherwise, ``fa2.py:656-657``).  Passing them allows a decode launch to
-      split keys across workgroups, as in the reference; the partials themselves live in a
-      private workspace (or ``workspace=``) with this library's own layout, and the contents of
-      ``partial_*`` are left unspecified.
+      split keys across workgroups, as in the reference; the partials themselves live in
+      ``workspace=`` (or the library's static scratch) with this library's own layout, and the
+      contents of ``partial_*`` are left unspecified.
     * ``use_grouped_query_tile``, ``warp_specialize``, ``is_hopper``: tuning knobs of the Triton
       kernel; accepted and ignored (the GQA group is always packed).
     * ``use_fp32_dot`` (``fa2.py:85-88``): ``False`` rounds a wider query to the cache's 16-bit type
@@ -229,21 +241,37 @@ def flash_attention(
     * ``scale`` (1.0, ``fa2.py:89``); ``query_window`` (None = anchored window; an int hides keys with
       ``q_pos - k_pos >= query_window`` as ``scripts/reference_impl.py:440-441`` does);
       ``window_sizes`` (``[B]`` int32 per-slot ``ctx_window_size``); ``workspace`` (uint8 tensor
-      used for split partials instead of the private one; ``False`` = use none and never split; ``"static"`` = the
-      library's built-in scratch array through ``g4b_attn_forward_static_scratch``, which allocates nothing and
-      refuses launches whose partials exceed ``g4b_static_scratch_bytes()``; calls that overlap on one GPU must not
-      share it); ``num_workers``; ``kernel_mask`` (profiling:
+      holding the split partials of this call -- size it with :func:`workspace_bytes` next to the engine's
+      ``fa_gqa_partial_o`` (``g4b/models/gemma4e.py:819-821``); ``None`` or ``"static"`` = the library's built-in
+      scratch array through ``g4b_attn_forward_static_scratch``: nothing is allocated, a launch whose partials exceed
+      ``g4b_static_scratch_bytes()`` runs unsplit, and calls that overlap on one GPU (two streams) must not share it,
+      so give every stream but one a workspace of its own; ``False`` = no scratch, never split); ``num_workers``; ``kernel_mask`` (profiling:
       bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
+    * ``decode_q``, ``decode_o`` (``[B, H, 1, D]``), ``decode_phase``: a mixed step in one launch.  The reference
+      serves a step that holds prefill-phase and decode-phase slots with two calls over the same batch tensors,
+      because its kernel skips per slot on ``user_phase[b] != PHASE`` (``fa2.py:332-335``), and its scheduler avoids
+      such steps (``g4b/scheduler.py:66,96-98``).  With these two tensors given, this call (the chunk: ``q``, ``o``,
+      ``phase``) also computes ``decode_o`` from ``decode_q`` for the slots in ``decode_phase``, in the same grid:
+      the chunk's workgroups and the decode stream's run on different compute units at the same time.  Same results
+      as the two calls.  ``workspace`` must then be a tensor of :func:`mixed_workspace_bytes` bytes (or absent: no
+      half splits its keys).  Head dimension 256.
 
     Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
     ignore (``g4b/models/gemma4e.py:593-607``).
     """
-    a, _keep, entry = _bind(
-        q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, partial_o, partial_l, partial_m,
+    kw = dict(
         use_grouped_query_tile=use_grouped_query_tile, warp_specialize=warp_specialize, is_hopper=is_hopper,
         use_fp32_dot=use_fp32_dot, stage=stage, scale=scale, query_window=query_window, window_sizes=window_sizes,
-        workspace=workspace, num_workers=num_workers, kernel_mask=kernel_mask,
+        num_workers=num_workers, kernel_mask=kernel_mask,
     )
+    if decode_q is not None or decode_o is not None:
+        if partial_o is not None or partial_l is not None or partial_m is not None:
+            raise ValueError("a mixed launch takes its scratch through workspace=, not partial_o/l/m")
+        a, _keep, entry = _bind_mixed(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase,
+                                      decode_q, decode_o, decode_phase, workspace, **kw)
+    else:
+        a, _keep, entry = _bind(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase,
+                                partial_o, partial_l, partial_m, workspace=workspace, **kw)
     _native.check(entry(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
     return None, None
 
@@ -270,5 +298,12 @@ class AttentionPlan:
 def plan_flash_attention(*args, **kwargs) -> AttentionPlan:
     """Same arguments as :func:`flash_attention` (without ``stream``); returns an :class:`AttentionPlan`."""
     kwargs.pop("stream", None)
-    a, keep, entry = _bind(*args, **kwargs)
+    if kwargs.get("decode_q") is not None or kwargs.get("decode_o") is not None:
+        decode_q, decode_o = kwargs.pop("decode_q", None), kwargs.pop("decode_o", None)
+        decode_phase = kwargs.pop("decode_phase", PHASE_DECODE)
+        workspace = kwargs.pop("workspace", None)
+        a, keep, entry = _bind_mixed(*args[:8], decode_q, decode_o, decode_phase, workspace, **kwargs)
+    else:
+        kwargs.pop("decode_q", None), kwargs.pop("decode_o", None), kwargs.pop("decode_phase", None)
+        a, keep, entry = _bind(*args, **kwargs)
     return AttentionPlan(a, keep, entry)

@@ -129,6 +129,24 @@ uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, i
 int32_t g4b_attn_default_workers(void);
 
 /*
+ * g4b_attn_forward_mixed: one launch for a step that holds prefill-phase and decode-phase slots at once.  The
+ * reference kernel skips per slot on user_phase[b] != PHASE (g4b/kernels/fa2.py:332-335), so such a step is two
+ * flash_attention calls over the same batch tensors, one per phase, and its scheduler avoids the case altogether
+ * (g4b/scheduler.py:66,96-98).  Here both calls are one grid: `prefill` is the argument block of the call whose query
+ * block is a chunk ((H/G)*Tq > 16), `decode` the block of the call with one (or a few) query tokens per slot
+ * ((H/G)*Tq <= 16); they must name the same caches, time_dim_sizes, user_phase, window_sizes, B, H, G, D, KV_CTX, cache
+ * dtype and ctx_window_size and differ in q, o, Tq, strides and phase.  Results are those of the two calls.  The
+ * workgroups of the two halves are dealt to different compute units, so the chunk's matrix work runs under the decode
+ * stream's memory time.  Head dimension 256.
+ *   workspace     one buffer for both halves, passed in `prefill->workspace` (`decode->workspace` is ignored), at
+ *                 least g4b_attn_mixed_workspace_bytes(...) bytes; NULL = neither half splits keys.
+ *   num_workers   `decode->num_workers`: 0 = the library's share-out of the chip between the halves.
+ */
+int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* decode, void* stream);
+uint64_t g4b_attn_mixed_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq_prefill, int32_t Tq_decode, int32_t D,
+                                        int32_t KV_CTX, int32_t ctx_window_size, int32_t has_window_sizes, int32_t num_workers);
+
+/*
  * g4b_attn_forward_static_scratch: g4b_attn_forward for callers that cannot allocate.  It has no counterpart in the
  * reference; it is for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc, which
  * have no place to get the split-KV workspace from.  Same arguments and results as g4b_attn_forward with a workspace

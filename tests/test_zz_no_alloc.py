@@ -77,9 +77,12 @@ def test_rejects_what_does_not_fit_and_a_foreign_workspace(fa):
     lib = _native.load()
     B, H, G, D, W = 2, 8, 2, 256, 512
     q, k, v, o = make_case(B, H, G, 1, D, W, seed=9)
-    args, keep, entry = fa._bind(q, k, v, o, i32([W, W]), u8([2, 2]), W, 2, *partials(4, B, H, 1, D), workspace="static",
-                                 num_workers=1 << 20)
-    assert entry is lib.g4b_attn_forward_static_scratch or entry == lib.g4b_attn_forward_static_scratch
+    args, keep, entry = fa._bind(q, k, v, o, i32([W, W]), u8([2, 2]), W, 2, *partials(4, B, H, 1, D), workspace="static")
+    assert C.cast(entry, C.c_void_p).value == C.cast(lib.g4b_attn_forward_static_scratch, C.c_void_p).value
+    # the wrapper runs a launch unsplit when its partials would not fit; the entry point itself refuses it
+    _, _, entry_big = fa._bind(q, k, v, o, i32([W, W]), u8([2, 2]), W, 2, *partials(4, B, H, 1, D), num_workers=1 << 20)
+    assert C.cast(entry_big, C.c_void_p).value == C.cast(lib.g4b_attn_forward, C.c_void_p).value
+    args.num_workers = 1 << 20
     rc = lib.g4b_attn_forward_static_scratch(C.byref(args), None)
     assert rc == _native.G4B_ERR_WORKSPACE, rc
     assert "static scratch holds" in _native.last_error()

@@ -366,7 +366,7 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
     g4b::MixedPlan mp = m.plan;
     mp.npx = (g4b::prefill_grid(pp) + 7) / 8;
     mp.combine_pf = g4b::prefill_combine_grid(pp);
-    mp.combine_dec = pair ? 0 : a->B * a->G * pd.R * pd.Tq;
+    mp.combine_dec = (pair || !m.nw) ? 0 : a->B * a->G * pd.R * pd.Tq;
     if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
     const hipError_t e = a->kv_dtype == G4B_DT_F16
                              ? g4b::launch_attn_mixed_f16(pp, pd, mp, a->D, static_cast<hipStream_t>(stream))

@@ -24,7 +24,8 @@ static hipError_t launch_decode_t(const AttnParams& p, hipStream_t stream) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (p.kernel_mask & 2) hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G, p.R * p.Tq), dim3(256), 0, stream, p);
+    // without a workspace every pair belongs to one wave, which also writes the zeros of an empty slot: nothing to merge
+    if ((p.kernel_mask & 2) && p.NW > 0) hipLaunchKernelGGL((attn_decode_combine<D>), dim3(p.B * p.G, p.R * p.Tq), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -278,7 +278,18 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
         if (w >= B * G) return;
         const int bb = w / G, g = w % G;
         const int tlb = slot_tiles(p, bb);
-        if (tlb > 0) decode_segment<D, CL, T, DH, QS>(p, w, bb, g, 0, tlb, tlb, xch);
+        if (tlb > 0) {
+            decode_segment<D, CL, T, DH, QS>(p, w, bb, g, 0, tlb, tlb, xch);
+        } else if (slot_info(p, bb).active && (DH == 1 || threadIdx.x < 64)) {  // one wave of the worker
+            // in-phase slot without any visible key: defined as zeros (no merge kernel runs on this path)
+            const int NR = p.R * p.Tq;
+            for (int idx = lane; idx < NR * (D / 4); idx += 64) {
+                const int row = idx / (D / 4), c4 = idx % (D / 4);
+                const int64_t ooff = (int64_t)bb * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] +
+                                     (int64_t)(row % p.Tq) * p.o_s[2];
+                store4(p.o, ooff + c4 * 4, p.o_dt, f4{0.f, 0.f, 0.f, 0.f});
+            }
+        }
         return;
     }
 

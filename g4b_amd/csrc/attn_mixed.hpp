@@ -5,7 +5,7 @@
 // number of compute units it gets; the decode stream is bound by HBM and reaches its full rate with a wave on about
 // a third of the SIMDs (384 single-wave workers read as fast as 1024).  Launched one after the other, each half
 // leaves the other's resource idle.  Here one grid carries both: workgroup ids are dealt so that every XCD gets the
-// same mix, `npx` prefill workgroups per XCD first and the decode workgroups after them; a prefill workgroup runs the
+// same mix, the decode workgroups first and `npx` prefill workgroups per XCD after them; a prefill workgroup runs the
 // body of the prefill kernel, a decode workgroup is four single-wave workers of the streaming kernel (or one
 // (slot, kv head) pair of the short-window variant).  Both kinds occupy a compute unit alone (registers, LDS), so
 // the hardware places prefill and decode workgroups side by side on different units and the chunk's matrix work runs
@@ -22,11 +22,13 @@ __global__ __launch_bounds__(256) void attn_mixed_kernel(const AttnParams pp, co
     extern __shared__ __align__(16) char smem[];
     __shared__ int sh_scan[8];
     const int x = blockIdx.x & 7, j = blockIdx.x >> 3;  // workgroups go to the XCDs round-robin by id
-    if (j < mp.npx) {
-        prefill_body<D, T, QS>(pp, j * 8 + x, smem, sh_scan);
+    const int ndx = (mp.nd_blocks + 7) >> 3;
+    if (j >= ndx) {
+        // the prefill grid is sized for every slot being in the prefill phase; the surplus leaves at once
+        prefill_body<D, T, QS>(pp, (j - ndx) * 8 + x, smem, sh_scan);
         return;
     }
-    const int d = (j - mp.npx) * 8 + x;
+    const int d = j * 8 + x;
     if (d >= mp.nd_blocks) return;
     if (mp.pair_path) {
         decode_pair_body<D, CL, T, QS>(pd, d, reinterpret_cast<float*>(smem));

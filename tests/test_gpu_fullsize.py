@@ -1,7 +1,8 @@
 """Parity at the full sizes of the five benchmark configurations.
 
-The fp64 oracle is evaluated on sampled slots / query rows so that it finishes in seconds; in
-addition, size-independent properties are checked on the whole output: split and unsplit launches
+The fp64 oracle is evaluated on sampled slots / query rows so that it finishes in seconds; every element of the
+large configurations (3a, 3b, 4, 5) is compared with the fp32 CPU restatement of the reference's attention as well
+(the tests at the end of this file); in addition, size-independent properties are checked on the whole output: split and unsplit launches
 agree, the anchored and the per-query window coincide where they must, uniform attention (K = 0)
 returns the mean of the visible V rows, and a launch is idempotent.
 """
@@ -222,3 +223,66 @@ def test_config5_mixed_step_two_launches_per_layer(fa):
         assert_close(op[32].float().cpu().numpy()[:, rows], oracle_rows(qp, k, v, 32, rows, tds[32], W, t), what=f"{name} chunk")
         for b in (0, 5, 17, 31):
             assert_close(od[b].float().cpu().numpy(), oracle_rows(qd, k, v, b, [0], tds[b], W, 1), what=f"{name} decode slot {b}")
+
+
+# ---- every output element of the large configurations against the CPU restatement of the reference ----------------
+# The fp64 oracle above is affordable on sampled rows only.  The fp32 torch-CPU restatement of the reference's own
+# attention (scripts/reference_impl.py:434-443, oracle.attention_ref.attention_cpu_baseline, query rows in blocks of
+# 512 so that the score tensor stays small) finishes the full configurations in seconds to tens of seconds, so every
+# element is compared with it as well, at the north-star tolerance widened by 2e-5 for the fp32 sums of the CPU path
+# itself (up to 32768 terms of magnitude <= 1 per row).
+CPU_FP32_SLACK = 2e-5
+
+
+def _cpu_reference(q, k, v, tds, phase, W, phase_id, **kw):
+    from oracle import attention_ref as ar
+
+    torch.set_num_threads(min(torch.get_num_threads(), 16))
+    return ar.attention_cpu_baseline(q.cpu(), k.cpu(), v.cpu(), tds, phase, W, phase_id, scale=SCALE, row_block=512, **kw).numpy()
+
+
+@pytest.mark.parametrize("qw", [None, 512], ids=["config3b_causal", "config3a_swa512"])
+def test_config3_prefill_8192_every_element(fa, qw):
+    S = 8192
+    q, k, v = randn16((1, H, S, D), 1), randn16((1, G, S, D), 2), randn16((1, G, S, D), 3)
+    o = torch.full_like(q, 777.0)
+    fa.flash_attention(q, k, v, o, i32([S]), u8([1]), S, 1, scale=SCALE, query_window=qw)
+    torch.cuda.synchronize()
+    ref = _cpu_reference(q, k, v, [S], [1], S, 1, query_window=qw)
+    assert_close(o.float().cpu().numpy(), ref, atol=2e-3 + CPU_FP32_SLACK, what=f"config 3 qw={qw}, all {H * S} rows")
+
+
+def test_config4_batched_decode_every_element(fa):
+    B, kv_ctx = 64, 32768
+    rng = np.random.default_rng(0)
+    tds = rng.integers(128, 32768 + 1, B).tolist()
+    win = [512 if b % 2 == 0 else kv_ctx for b in range(B)]
+    q, k, v = randn16((B, H, 1, D), 1), randn16((B, G, kv_ctx, D), 2), randn16((B, G, kv_ctx, D), 3)
+    ws = torch.empty(fa.workspace_bytes(B, H, G, 1, D), dtype=torch.uint8, device="cuda")
+    o = torch.full_like(q, 777.0)
+    fa.flash_attention(q, k, v, o, i32(tds), u8([2] * B), kv_ctx, 2, scale=SCALE, window_sizes=i32(win), workspace=ws)
+    torch.cuda.synchronize()
+    ref = _cpu_reference(q, k, v, tds, [2] * B, kv_ctx, 2, window_sizes=win)
+    assert_close(o.float().cpu().numpy(), ref, atol=2e-3 + CPU_FP32_SLACK, what="config 4, all 64 slots")
+
+
+def test_config5_mixed_step_one_launch_every_element(fa):
+    """Configuration 5 at full size through the one-launch mixed mode, both layer kinds, every element of both halves."""
+    B, t, ctx = 33, 512, 16384
+    rng = np.random.default_rng(0)
+    tds = rng.integers(1024, 16384 + 1, 32).tolist() + [ctx + t]
+    phase = [2] * 32 + [1]
+    qp, qd = randn16((B, H, t, D), 1), randn16((B, H, 1, D), 2)
+    for W, T in ((32768, 32768 + t - 1), (512, 512 + t - 1)):
+        k, v = randn16((B, G, T, D), 3), randn16((B, G, T, D), 4)
+        ws = torch.empty(fa.mixed_workspace_bytes(B, H, G, t, 1, D, T, W), dtype=torch.uint8, device="cuda")
+        op, od = torch.full_like(qp, 777.0), torch.full_like(qd, 777.0)
+        fa.flash_attention(qp, k, v, op, i32(tds), u8(phase), W, 1, scale=SCALE, workspace=ws, decode_q=qd, decode_o=od)
+        torch.cuda.synchronize()
+        ref_p = _cpu_reference(qp[32:], k[32:], v[32:], tds[32:], [1], W, 1)
+        assert_close(op[32:].float().cpu().numpy(), ref_p, atol=2e-3 + CPU_FP32_SLACK, what=f"config 5 chunk, W={W}")
+        assert (op[:32] == 777.0).all()
+        ref_d = _cpu_reference(qd, k, v, tds, phase, W, 2)
+        assert_close(od[:32].float().cpu().numpy(), ref_d[:32], atol=2e-3 + CPU_FP32_SLACK, what=f"config 5 decode, W={W}")
+        assert (od[32:] == 777.0).all()
+        del k, v

@@ -559,7 +559,9 @@ def measure(wl: Workload, steps: int, warmup: int):
         floor_ms = (wl.bytes / (HBM_PEAK_GBPS * 1e9) + wl.flops / (FP16_PEAK_TFLOPS * 1e12)) * 1e3
         res["roofline"] = {"bound": "hbm+mfma", "decode_bytes": wl.bytes, "prefill_flops": wl.flops,
                            "floor_ms": round(floor_ms, 4), "kernel_ms": round(k_avg, 4),
-                           "frac": round(floor_ms / k_avg, 4), "traffic": measured_traffic_bytes(wl.key)}
+                           "frac": round(floor_ms / k_avg, 4),
+                           # the counters give the main kernel's average bytes per dispatch over both layer kinds
+                           "traffic": None if measured_traffic_bytes(wl.key) is None else measured_traffic_bytes(wl.key) * wl.layers}
     return res
 
 

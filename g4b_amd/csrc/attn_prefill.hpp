@@ -70,17 +70,148 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     nth_active_slot(p, -1, n_active, sh_scan);
     if (n_active == 0) return;
     const int nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
-    const PfMap map = pf_map(n_active * p.G * nsplit, (Tq + TOKB - 1) / TOKB);
+    const int nq_tiles = (Tq + TOKB - 1) / TOKB;
+    const PfMap map = pf_map(n_active * p.G * nsplit, pf_ranks(nsplit, nq_tiles));
     if (bid >= map.grid) return;
     int head, rank;
     pf_item(map, bid, head, rank);
     if (rank >= map.nq) return;
-    const int qtile = map.nq - 1 - rank;
+    // Unsplit launches give a workgroup two query tiles of its head, the rank-th from the end and the rank-th from the
+    // start: under the causal mask their key ranges add up to the same length for every workgroup, and the second
+    // item starts without a new workgroup having to be placed, scan the slots and set its staging up.
+    const int ipw = pf_items_per_workgroup(nsplit, nq_tiles);
+    const int qtile_first = nq_tiles - 1 - rank;
+    const int n_items = (ipw == 2 && rank != qtile_first) ? 2 : 1;
     const int split = head % nsplit, g = (head / nsplit) % p.G, a_idx = head / (nsplit * p.G);
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);  // workgroup-uniform
 
     const SlotInfo si = slot_info(p, b);
 
+    const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
+    const char* vbase = static_cast<const char*>(p.v) + ((int64_t)b * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
+    auto key_off = [&](int j) -> uint32_t {  // byte offset of logical key j (clamped to the window) in the ring
+        j = min(max(j, 0), si.window - 1);
+        int r = si.ring_start + j;
+        r = (r >= KV_CTX) ? r - KV_CTX : r;
+        return (uint32_t)r * (uint32_t)SM::ROW;
+    };
+
+    // ---- staging ------------------------------------------------------------------------------------------
+    // LDS map: K stages at [0, 2*TILE), V stages at [2*TILE, 4*TILE).  Wave `wave` moves chunks
+    // wave*CHUNKS .. +CHUNKS of each tile; chunk c covers bytes [c*1024, +1024) of the tile, lane l its piece l.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the dynamic segment
+    const int st_row_in_chunk = lane / PIECES;        // 0 .. ROWS_PER_CHUNK-1
+    const int st_piece_lds = lane % PIECES;           // 16-byte piece position inside the LDS row
+    auto st_row = [&](int i) { return (wave * CHUNKS + i) * ROWS_PER_CHUNK + st_row_in_chunk; };
+    auto k_piece = [&](int row) { return st_piece_lds ^ (row & 15); };
+    auto v_piece = [&](int row) { return st_piece_lds ^ (4 * (row & SM::VSWZ)); };
+    // A tile is "plain" when its 64 keys lie inside the window and do not straddle the ring seam: then its rows
+    // are consecutive in memory and every lane's source offset is a loop constant added to one scalar base.
+    // Only the first / last tiles of a slot and the one on the seam take the general path with per-row clamping.
+    uint32_t k_const[CHUNKS], v_const[CHUNKS];
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+        const int row = st_row(i);
+        // chunk i is issued with instruction offset (i % 4) KiB, which moves source and destination alike
+        k_const[i] = (uint32_t)row * SM::ROW + (uint32_t)k_piece(row) * 16u - (uint32_t)(i & 3) * 1024u;
+        v_const[i] = (uint32_t)row * SM::ROW + (uint32_t)v_piece(row) * 16u - (uint32_t)(i & 3) * 1024u;
+    }
+    auto plain_row0 = [&](int kt) -> int {  // ring row of the tile's first key, or -1
+        const int jb = kt * PF_BN;
+        if (jb + PF_BN > si.window) return -1;
+        int r0 = si.ring_start + jb;
+        r0 = (r0 >= KV_CTX) ? r0 - KV_CTX : r0;
+        return (r0 + PF_BN <= KV_CTX) ? r0 : -1;
+    };
+    // Source of K or V tile kt as scalar base + per-lane byte offsets (the instruction offset of chunk i comes on
+    // top: on the general path the base is lowered by 3 KiB so that the lane offsets stay non-negative).
+    auto tile_src = [&](int kt, bool is_v, const char*& src, uint32_t(&ofs)[CHUNKS]) {
+        const int r0 = plain_row0(kt);
+        const char* base = is_v ? vbase : kbase;
+        if (r0 >= 0) {
+            src = base + (int64_t)r0 * SM::ROW;
+#pragma unroll
+            for (int i = 0; i < CHUNKS; ++i) ofs[i] = is_v ? v_const[i] : k_const[i];
+        } else {
+            src = base - 3072;
+#pragma unroll
+            for (int i = 0; i < CHUNKS; ++i) {
+                const int row = st_row(i);
+                ofs[i] = key_off(kt * PF_BN + row) + (uint32_t)(is_v ? v_piece(row) : k_piece(row)) * 16u + 3072u -
+                         (uint32_t)(i & 3) * 1024u;
+            }
+        }
+    };
+    const uint32_t wave_chunk0 = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (CHUNKS * 1024);
+    // chunk i of a tile: four chunks share one M0 base
+    auto dma_chunk = [&](int i, const char* src, const uint32_t(&ofs)[CHUNKS], uint32_t dst) {
+        if ((i & 3) == 0) dma_set_base(dst + i * 1024);
+        if ((i & 3) == 0) dma16_to_lds_at<0>(src, ofs[i]);
+        if ((i & 3) == 1) dma16_to_lds_at<1024>(src, ofs[i]);
+        if ((i & 3) == 2) dma16_to_lds_at<2048>(src, ofs[i]);
+        if ((i & 3) == 3) dma16_to_lds_at<3072>(src, ofs[i]);
+    };
+    auto stage_whole_tile = [&](int kt, bool is_v, int stage) {  // prologue only: all chunks at once
+        const char* src;
+        uint32_t ofs[CHUNKS];
+        tile_src(kt, is_v, src, ofs);
+        const uint32_t dst = lds0 + (is_v ? 2 * SM::TILE : 0) + stage * SM::TILE + wave_chunk0;
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) dma_chunk(i, src, ofs, dst);
+    };
+
+    // ---- operand read offsets (bytes from the start of a stage pair) ----------------------------------------
+    // K^T step (mt, c): row mt*32 + n32, piece 2c + h2, swizzled with (row & 15) = (n32 & 15)
+    uint32_t koff[8];
+#pragma unroll
+    for (int c8 = 0; c8 < 8; ++c8) koff[c8] = (uint32_t)n32 * SM::ROW + (uint32_t)(((2 * c8 + h2) ^ (n32 & 15)) * 16);
+    // V^T fragment of step (cu, dt): d = 32dt + n32, keys {16cu + 4h2 + 0..3, 16cu + 8 + 4h2 + 0..3} (the order in
+    // which this lane half holds P), fetched with two transposing reads.  Inside a 16-lane group, lane 4r + q
+    // points at columns 4q..4q+3 of key r of the block and receives the group's column (lane % 16) of 4 keys.
+    const int tr_r = (lane & 15) >> 2, tr_q = lane & 3, tr_dhalf = (lane >> 4) & 1;
+    const int tr_key = 4 * h2 + tr_r;  // key (mod 16) this lane points at
+    uint32_t voff[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int piece = dt * 4 + tr_dhalf * 2 + (tr_q >> 1);
+        voff[dt] = 2 * SM::TILE + (uint32_t)tr_key * SM::ROW + (uint32_t)((piece ^ (4 * (tr_key & SM::VSWZ))) * 16) +
+                   (uint32_t)(tr_q & 1) * 8u;
+    }
+    // Operand reads are issued as volatile asm, PF_PD steps ahead of the MFMA that consumes them, and
+    // retired with explicit lgkmcnt waits: LDS returns data in order, so "at most n outstanding" is exact
+    // for the oldest read whatever else the compiler has in flight.
+    uint32_t kaddr[8], vaddr[DT];
+    auto k_issue = [&](int idx) -> u4 {  // needs kaddr[] of the stage
+        const int c = idx >> 1, mt = idx & 1;
+        return lds_read16(kaddr[c & 7], mt * 32 * SM::ROW + (c >> 3) * 256);
+    };
+    struct VFrag {
+        u2 lo, hi;
+    };
+    auto v_issue = [&](int idx) -> VFrag {  // needs vaddr[] of the stage
+        const int cu = idx / DT, dt = idx % DT;
+        VFrag f;
+        f.lo = lds_read8_tr16(vaddr[dt], cu * 16 * SM::ROW);
+        f.hi = lds_read8_tr16(vaddr[dt], (cu * 16 + 8) * SM::ROW);
+        return f;
+    };
+    // Reads are retired a pair at a time; `left` = pairs of the same sequence issued after the one being retired
+    // (a constant after unrolling).
+    auto wait_pair = [&](u4& a0, u4& a1, int left) {
+        if (left >= 2) lds_wait_pair<4>(a0, a1);
+        else if (left == 1) lds_wait_pair<2>(a0, a1);
+        else lds_wait_pair<0>(a0, a1);
+    };
+    auto wait_pair2 = [&](VFrag& f0, VFrag& f1, int left) {  // every fragment is two reads
+        if (left >= 2) lds_wait4<8>(f0.lo, f0.hi, f1.lo, f1.hi);
+        else if (left == 1) lds_wait4<4>(f0.lo, f0.hi, f1.lo, f1.hi);
+        else lds_wait4<0>(f0.lo, f0.hi, f1.lo, f1.hi);
+    };
+#pragma unroll
+    for (int item = 0; item < 2; ++item) {
+    if (item >= n_items) break;
+    if (item > 0) __syncthreads();  // every wave has read its rows of the previous item back from LDS
+    const int qtile = item == 0 ? qtile_first : rank;
     const int tok0 = qtile * TOKB;
     const int tok_last = min(tok0 + TOKB, Tq) - 1;
     // key range of the workgroup and the range that every row shares
@@ -106,127 +237,6 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     float m_run = -INFINITY, l_run = 0.f;  // exponent reference in log2 units (scaled), running sum (this lane's keys)
 
     if (hi_wg > lo_wg) {
-        const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
-        const char* vbase = static_cast<const char*>(p.v) + ((int64_t)b * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
-        auto key_off = [&](int j) -> uint32_t {  // byte offset of logical key j (clamped to the window) in the ring
-            j = min(max(j, 0), si.window - 1);
-            int r = si.ring_start + j;
-            r = (r >= KV_CTX) ? r - KV_CTX : r;
-            return (uint32_t)r * (uint32_t)SM::ROW;
-        };
-
-        // ---- staging ------------------------------------------------------------------------------------------
-        // LDS map: K stages at [0, 2*TILE), V stages at [2*TILE, 4*TILE).  Wave `wave` moves chunks
-        // wave*CHUNKS .. +CHUNKS of each tile; chunk c covers bytes [c*1024, +1024) of the tile, lane l its piece l.
-        const uint32_t lds0 = (uint32_t)(uintptr_t)smem;  // LDS byte address of the dynamic segment
-        const int st_row_in_chunk = lane / PIECES;        // 0 .. ROWS_PER_CHUNK-1
-        const int st_piece_lds = lane % PIECES;           // 16-byte piece position inside the LDS row
-        auto st_row = [&](int i) { return (wave * CHUNKS + i) * ROWS_PER_CHUNK + st_row_in_chunk; };
-        auto k_piece = [&](int row) { return st_piece_lds ^ (row & 15); };
-        auto v_piece = [&](int row) { return st_piece_lds ^ (4 * (row & SM::VSWZ)); };
-        // A tile is "plain" when its 64 keys lie inside the window and do not straddle the ring seam: then its rows
-        // are consecutive in memory and every lane's source offset is a loop constant added to one scalar base.
-        // Only the first / last tiles of a slot and the one on the seam take the general path with per-row clamping.
-        uint32_t k_const[CHUNKS], v_const[CHUNKS];
-#pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) {
-            const int row = st_row(i);
-            // chunk i is issued with instruction offset (i % 4) KiB, which moves source and destination alike
-            k_const[i] = (uint32_t)row * SM::ROW + (uint32_t)k_piece(row) * 16u - (uint32_t)(i & 3) * 1024u;
-            v_const[i] = (uint32_t)row * SM::ROW + (uint32_t)v_piece(row) * 16u - (uint32_t)(i & 3) * 1024u;
-        }
-        auto plain_row0 = [&](int kt) -> int {  // ring row of the tile's first key, or -1
-            const int jb = kt * PF_BN;
-            if (jb + PF_BN > si.window) return -1;
-            int r0 = si.ring_start + jb;
-            r0 = (r0 >= KV_CTX) ? r0 - KV_CTX : r0;
-            return (r0 + PF_BN <= KV_CTX) ? r0 : -1;
-        };
-        // Source of K or V tile kt as scalar base + per-lane byte offsets (the instruction offset of chunk i comes on
-        // top: on the general path the base is lowered by 3 KiB so that the lane offsets stay non-negative).
-        auto tile_src = [&](int kt, bool is_v, const char*& src, uint32_t(&ofs)[CHUNKS]) {
-            const int r0 = plain_row0(kt);
-            const char* base = is_v ? vbase : kbase;
-            if (r0 >= 0) {
-                src = base + (int64_t)r0 * SM::ROW;
-#pragma unroll
-                for (int i = 0; i < CHUNKS; ++i) ofs[i] = is_v ? v_const[i] : k_const[i];
-            } else {
-                src = base - 3072;
-#pragma unroll
-                for (int i = 0; i < CHUNKS; ++i) {
-                    const int row = st_row(i);
-                    ofs[i] = key_off(kt * PF_BN + row) + (uint32_t)(is_v ? v_piece(row) : k_piece(row)) * 16u + 3072u -
-                             (uint32_t)(i & 3) * 1024u;
-                }
-            }
-        };
-        const uint32_t wave_chunk0 = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (CHUNKS * 1024);
-        // chunk i of a tile: four chunks share one M0 base
-        auto dma_chunk = [&](int i, const char* src, const uint32_t(&ofs)[CHUNKS], uint32_t dst) {
-            if ((i & 3) == 0) dma_set_base(dst + i * 1024);
-            if ((i & 3) == 0) dma16_to_lds_at<0>(src, ofs[i]);
-            if ((i & 3) == 1) dma16_to_lds_at<1024>(src, ofs[i]);
-            if ((i & 3) == 2) dma16_to_lds_at<2048>(src, ofs[i]);
-            if ((i & 3) == 3) dma16_to_lds_at<3072>(src, ofs[i]);
-        };
-        auto stage_whole_tile = [&](int kt, bool is_v, int stage) {  // prologue only: all chunks at once
-            const char* src;
-            uint32_t ofs[CHUNKS];
-            tile_src(kt, is_v, src, ofs);
-            const uint32_t dst = lds0 + (is_v ? 2 * SM::TILE : 0) + stage * SM::TILE + wave_chunk0;
-#pragma unroll
-            for (int i = 0; i < CHUNKS; ++i) dma_chunk(i, src, ofs, dst);
-        };
-
-        // ---- operand read offsets (bytes from the start of a stage pair) ----------------------------------------
-        // K^T step (mt, c): row mt*32 + n32, piece 2c + h2, swizzled with (row & 15) = (n32 & 15)
-        uint32_t koff[8];
-#pragma unroll
-        for (int c8 = 0; c8 < 8; ++c8) koff[c8] = (uint32_t)n32 * SM::ROW + (uint32_t)(((2 * c8 + h2) ^ (n32 & 15)) * 16);
-        // V^T fragment of step (cu, dt): d = 32dt + n32, keys {16cu + 4h2 + 0..3, 16cu + 8 + 4h2 + 0..3} (the order in
-        // which this lane half holds P), fetched with two transposing reads.  Inside a 16-lane group, lane 4r + q
-        // points at columns 4q..4q+3 of key r of the block and receives the group's column (lane % 16) of 4 keys.
-        const int tr_r = (lane & 15) >> 2, tr_q = lane & 3, tr_dhalf = (lane >> 4) & 1;
-        const int tr_key = 4 * h2 + tr_r;  // key (mod 16) this lane points at
-        uint32_t voff[DT];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const int piece = dt * 4 + tr_dhalf * 2 + (tr_q >> 1);
-            voff[dt] = 2 * SM::TILE + (uint32_t)tr_key * SM::ROW + (uint32_t)((piece ^ (4 * (tr_key & SM::VSWZ))) * 16) +
-                       (uint32_t)(tr_q & 1) * 8u;
-        }
-        // Operand reads are issued as volatile asm, PF_PD steps ahead of the MFMA that consumes them, and
-        // retired with explicit lgkmcnt waits: LDS returns data in order, so "at most n outstanding" is exact
-        // for the oldest read whatever else the compiler has in flight.
-        uint32_t kaddr[8], vaddr[DT];
-        auto k_issue = [&](int idx) -> u4 {  // needs kaddr[] of the stage
-            const int c = idx >> 1, mt = idx & 1;
-            return lds_read16(kaddr[c & 7], mt * 32 * SM::ROW + (c >> 3) * 256);
-        };
-        struct VFrag {
-            u2 lo, hi;
-        };
-        auto v_issue = [&](int idx) -> VFrag {  // needs vaddr[] of the stage
-            const int cu = idx / DT, dt = idx % DT;
-            VFrag f;
-            f.lo = lds_read8_tr16(vaddr[dt], cu * 16 * SM::ROW);
-            f.hi = lds_read8_tr16(vaddr[dt], (cu * 16 + 8) * SM::ROW);
-            return f;
-        };
-        // Reads are retired a pair at a time; `left` = pairs of the same sequence issued after the one being retired
-        // (a constant after unrolling).
-        auto wait_pair = [&](u4& a0, u4& a1, int left) {
-            if (left >= 2) lds_wait_pair<4>(a0, a1);
-            else if (left == 1) lds_wait_pair<2>(a0, a1);
-            else lds_wait_pair<0>(a0, a1);
-        };
-        auto wait_pair2 = [&](VFrag& f0, VFrag& f1, int left) {  // every fragment is two reads
-            if (left >= 2) lds_wait4<8>(f0.lo, f0.hi, f1.lo, f1.hi);
-            else if (left == 1) lds_wait4<4>(f0.lo, f0.hi, f1.lo, f1.hi);
-            else lds_wait4<0>(f0.lo, f0.hi, f1.lo, f1.hi);
-        };
-
         // this workgroup's share of the item's key tiles
         int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
         if (nsplit > 1) {
@@ -477,6 +487,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
                 store4(p.o, off + pc * 4, p.o_dt, v);
             }
         }
+    }
     }
 }
 

@@ -380,7 +380,7 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
 template <class T, bool QS>
 static hipError_t launch_prefill_wide_t(const AttnParams& p, hipStream_t stream) {
     const int slots = p.part_o ? p.split_slots : 1;
-    const int blocks = prefill_grid(p, QS ? PW_BM / 2 : PW_BM);
+    const int blocks = prefill_grid(p, QS ? PW_BM / 2 : PW_BM, false);
     static uint64_t attr_done = 0;
     hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<T, QS>), PW_SMEM, attr_done);
     if (e != hipSuccess) return e;

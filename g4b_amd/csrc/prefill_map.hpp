@@ -43,15 +43,25 @@ __host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int&
     }
 }
 
+// Query tiles per workgroup of the 128/256 kernel.  A launch that does not split keys pairs the r-th heaviest query
+// tile of a head with the r-th lightest in one workgroup: equal work for every workgroup under the causal mask, and
+// half as many workgroup starts.
+__host__ __device__ inline int pf_items_per_workgroup(int nsplit, int nq) { return (nsplit == 1 && nq >= 2) ? 2 : 1; }
+// Ranks (workgroups) per head: query tiles, or pairs of them.
+__host__ __device__ inline int pf_ranks(int nsplit, int nq) {
+    return pf_items_per_workgroup(nsplit, nq) == 2 ? (nq + 1) / 2 : nq;
+}
+
 // Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on
-// the device and surplus workgroups leave at once.
-inline int prefill_grid(const AttnParams& p, int bm = PF_BM) {
+// the device and surplus workgroups leave at once.  paired: the kernel gives a workgroup pf_items_per_workgroup tiles.
+inline int prefill_grid(const AttnParams& p, int bm = PF_BM, bool paired = true) {
     const int tokb = bm / p.R;
     const int nq = (p.Tq + tokb - 1) / tokb;
     const int slots = p.part_o ? p.split_slots : 1;
     int blocks = 0;
     for (int n = 1; n <= p.B; ++n) {
-        const int g = pf_map(n * p.G * prefill_splits(slots, n), nq).grid;
+        const int ns = prefill_splits(slots, n);
+        const int g = pf_map(n * p.G * ns, paired ? pf_ranks(ns, nq) : nq).grid;
         blocks = g > blocks ? g : blocks;
     }
     return blocks;

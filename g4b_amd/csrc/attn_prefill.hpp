@@ -42,6 +42,11 @@ struct PfSmem {
     static constexpr int VSWZ = (D >= 256) ? 7 : 3;  // (V row & VSWZ) selects the 64-byte group swizzle
 };
 
+// The small pieces this kernel has in common with the head-dimension-512 kernel (work selection, ring arithmetic, edge
+// mask, lazy rescaling, chunk issue; prefill_common.hpp) are spelled out here on purpose: routed through the shared
+// helpers the compiler allocates the main loop's registers differently and the S = 8192 launch measured 2 to 4 %
+// slower on the same board, helper by helper.
+//
 // QS: the query is wider than the cache type (fp32 scratchpads over a 16-bit cache) and enters S^T = K Q^T as two
 // B operands, the rounded value and its rounding error, against the same K fragments.
 // The body of workgroup `bid` of a launch (256 threads).  smem: 4 * PfSmem<D>::TILE bytes of LDS, 16-byte aligned;

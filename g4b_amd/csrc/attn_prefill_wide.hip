@@ -21,7 +21,7 @@
 #include "common.hpp"
 #include "launch.hpp"
 #include "prefill_combine.hpp"
-#include "prefill_map.hpp"
+#include "prefill_common.hpp"
 
 namespace g4b {
 
@@ -60,20 +60,13 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
     constexpr int BM = 4 * WROWS;
     const int TOKB = BM / R;
     __shared__ int sh_scan[8];
-    int n_active;
-    nth_active_slot(p, -1, n_active, sh_scan);
-    if (n_active == 0) return;
-    const int nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
-    const PfMap map = pf_map(n_active * p.G * nsplit, (Tq + TOKB - 1) / TOKB);
-    if ((int)blockIdx.x >= map.grid) return;
-    int head, rank;
-    pf_item(map, blockIdx.x, head, rank);
-    if (rank >= map.nq) return;
-    const int qtile = map.nq - 1 - rank;
-    const int split = head % nsplit, g = (head / nsplit) % p.G, a_idx = head / (nsplit * p.G);
-    const int b = nth_active_slot(p, a_idx, n_active, sh_scan);  // workgroup-uniform
+    const PfWork work = pf_select_work(p, blockIdx.x, BM, false, sh_scan);
+    if (!work.valid) return;
+    const int nsplit = work.nsplit, qtile = work.nq_tiles - 1 - work.rank;  // heaviest (latest) query tiles first
+    const int split = work.split, g = work.g, a_idx = work.a_idx, b = work.b;
 
     const SlotInfo si = slot_info(p, b);
+    const PfRing ring{si.window, si.ring_start, KV_CTX, (uint32_t)ROW};
     const int tok0 = qtile * TOKB;
     const int tok_last = min(tok0 + TOKB, Tq) - 1;
     int lo_wg, hi_wg, lo_max, hi_min;
@@ -99,12 +92,6 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
     if (hi_wg > lo_wg) {
         const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
         const char* vbase = static_cast<const char*>(p.v) + ((int64_t)b * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
-        auto key_off = [&](int j) -> uint32_t {  // byte offset of logical key j (clamped to the window) in the ring
-            j = min(max(j, 0), si.window - 1);
-            int r = si.ring_start + j;
-            r = (r >= KV_CTX) ? r - KV_CTX : r;
-            return (uint32_t)r * (uint32_t)ROW;
-        };
 
         // ---- staging: K stages at [0, 2*TILE), V stages at [2*TILE, 4*TILE); wave w moves rows 8w .. 8w+7 of a tile,
         // lane l the 16-byte piece that lands at position l of the LDS row.  Source offsets are recomputed where they
@@ -112,19 +99,12 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
         const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
         const int wrow0 = wave * CHUNKS;
         auto src_piece = [&](int row, bool is_v) { return is_v ? (lane ^ (4 * (row & 7))) : (lane ^ (row & 15)); };
-        auto plain_row0 = [&](int kt) -> int {  // ring row of the tile's first key when its rows are consecutive, or -1
-            const int jb = kt * PW_BN;
-            if (jb + PW_BN > si.window) return -1;
-            int r0 = si.ring_start + jb;
-            r0 = (r0 >= KV_CTX) ? r0 - KV_CTX : r0;
-            return (r0 + PW_BN <= KV_CTX) ? r0 : -1;
-        };
         struct TileSrc {
             const char* src;  // scalar base
             int kt, plain;
         };
         auto tile_src = [&](int kt, bool is_v) -> TileSrc {
-            const int r0 = plain_row0(kt);
+            const int r0 = ring.plain_row0(kt * PW_BN, PW_BN);
             const char* base = is_v ? vbase : kbase;
             TileSrc t;
             t.kt = kt;
@@ -138,16 +118,11 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
             const int row = wrow0 + i;
             const uint32_t pc = (uint32_t)src_piece(row, is_v) * 16u;
             if (t.plain) return (uint32_t)row * ROW + pc - (uint32_t)(i & 3) * 1024u;
-            return key_off(t.kt * PW_BN + row) + pc + 3072u - (uint32_t)(i & 3) * 1024u;
+            return ring.key_off(t.kt * PW_BN + row) + pc + 3072u - (uint32_t)(i & 3) * 1024u;
         };
         const uint32_t wave_chunk0 = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * (CHUNKS * 1024);
         auto dma_chunk = [&](int i, const TileSrc& t, bool is_v, uint32_t dst) {
-            const uint32_t ofs = chunk_ofs(t, i, is_v);
-            if ((i & 3) == 0) dma_set_base(dst + i * 1024);
-            if ((i & 3) == 0) dma16_to_lds_at<0>(t.src, ofs);
-            if ((i & 3) == 1) dma16_to_lds_at<1024>(t.src, ofs);
-            if ((i & 3) == 2) dma16_to_lds_at<2048>(t.src, ofs);
-            if ((i & 3) == 3) dma16_to_lds_at<3072>(t.src, ofs);
+            pf_dma_chunk(i, t.src, chunk_ofs(t, i, is_v), dst);
         };
 
         // ---- operand read offsets --------------------------------------------------------------------------
@@ -257,11 +232,7 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
                 // ---- edge tiles: mask
                 const int jb = kt * PW_BN;
                 if ((jb < lo_max) || (jb + PW_BN > hi_min)) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int j = jb + 8 * (i >> 2) + 4 * h2 + (i & 3);
-                        if (j < lo_r || j >= hi_r) s[i] = -INFINITY;
-                    }
+                    pf_mask_block(s, jb, h2, lo_r, hi_r);
                 }
 
                 // ---- online softmax with lazy rescaling (the exponent reference moves only when the maximum outgrows
@@ -270,28 +241,7 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const AttnParams
 #pragma unroll
                 for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
                 mx = half_swap_max(mx) * p.c;
-                const bool grow = mx > m_run + PF_TAU;
-                if (__any(grow)) {
-                    const float m_new = grow ? mx : m_run;
-                    const float alpha = grow ? fast_exp2(m_run - mx) : 1.f;
-                    const bool touch = grow && (m_run != -INFINITY);
-                    m_run = m_new;
-                    l_run *= alpha;
-                    if (__any(touch)) {
-                        // the accumulators live in AGPRs: spell the read-scale-write out so the copies stay inside
-                        // this rarely taken branch
-#pragma unroll
-                        for (int i = 0; i < DT; ++i)
-#pragma unroll
-                            for (int j = 0; j < 16; ++j) {
-                                float t, r;
-                                asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[i][j]));
-                                t *= alpha;
-                                asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(r) : "v"(t));
-                                acc[i][j] = r;
-                            }
-                    }
-                }
+                G4B_PF_LAZY_RESCALE(acc, DT, m_run, l_run, mx);
                 const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
                 float psum = 0.f;
                 u4 pf[2];  // [16-key group] -> 8 keys of this lane half

@@ -335,13 +335,16 @@ class MixedStep(Workload):
 
     bound = "hbm"
 
-    def __init__(self, device, seed=0, layers=35, one_launch=True):
+    def __init__(self, device, seed=0, layers=35, one_launch=True, global_dim=D):
         import numpy as np
         import torch
 
         from g4b_amd.kernels import fa2
 
         self.name = "mixed_step_35_layers" if one_launch else "mixed_step_35_layers_two_launches"
+        if global_dim != D:
+            self.name += f"_global_d{global_dim}"  # Gemma-4's global-attention layers use head dimension 512
+        Dg = self.Dg = global_dim
         self.fa2 = fa2
         self.layers = layers
         self.one_launch = one_launch
@@ -355,29 +358,34 @@ class MixedStep(Workload):
         self.qp = _randn_f16((B, H, t, D), seed + 1, device)
         self.qd = _randn_f16((B, H, 1, D), seed + 2, device)
         self.op, self.od = torch.empty_like(self.qp), torch.empty_like(self.qd)
-        self.kg = _randn_f16((B, G, self.T_global, D), seed + 3, device)
-        self.vg = _randn_f16((B, G, self.T_global, D), seed + 4, device)
+        if Dg != D:  # the global layers' own scratchpads
+            self.qpg, self.qdg = _randn_f16((B, H, t, Dg), seed + 7, device), _randn_f16((B, H, 1, Dg), seed + 8, device)
+            self.opg, self.odg = torch.empty_like(self.qpg), torch.empty_like(self.qdg)
+        else:
+            self.qpg, self.qdg, self.opg, self.odg = self.qp, self.qd, self.op, self.od
+        self.kg = _randn_f16((B, G, self.T_global, Dg), seed + 3, device)
+        self.vg = _randn_f16((B, G, self.T_global, Dg), seed + 4, device)
         self.ks = _randn_f16((B, G, self.T_swa, D), seed + 5, device)
         self.vs = _randn_f16((B, G, self.T_swa, D), seed + 6, device)
         self.tds = torch.tensor(self.tds_list, dtype=torch.int32, device=device)
         self.phase = torch.tensor([2] * 32 + [1], dtype=torch.uint8, device=device)
-        self.ws = torch.empty(max(fa2.workspace_bytes(B, H, G, 1, D),
-                                  fa2.mixed_workspace_bytes(B, H, G, t, 1, D, self.T_global, self.W_global),
+        self.ws = torch.empty(max(fa2.workspace_bytes(B, H, G, 1, Dg), fa2.workspace_bytes(B, H, G, t, Dg),
+                                  fa2.mixed_workspace_bytes(B, H, G, t, 1, Dg, self.T_global, self.W_global),
                                   fa2.mixed_workspace_bytes(B, H, G, t, 1, D, self.T_swa, self.W_swa)),
                               dtype=torch.uint8, device=device)
         self.plans = {}
         n_swa, n_glob = (layers + 1) // 2, layers // 2
-        dec_g = 2 * G * D * 2 * sum(min(x, self.W_global) for x in dec_len)
+        dec_g = 2 * G * Dg * 2 * sum(min(x, self.W_global) for x in dec_len)
         dec_s = 2 * G * D * 2 * sum(min(x, self.W_swa) for x in dec_len)
         pre_g_pairs = t * ctx + t * (t + 1) // 2
         pre_s_pairs = t * (t + 1) // 2  # anchored window: a chunk of W tokens sees only itself
         self.bytes = n_glob * dec_g + n_swa * dec_s
-        self.flops = 4 * H * D * (n_glob * pre_g_pairs + n_swa * pre_s_pairs)
+        self.flops = 4 * H * (Dg * n_glob * pre_g_pairs + D * n_swa * pre_s_pairs)
         self.units = self.bytes
         self.detail = {
             "launches_per_layer": 1 if one_launch else 2,
             "decode_bytes_global_layer": dec_g, "decode_bytes_swa_layer": dec_s,
-            "prefill_flops_global_layer": 4 * H * D * pre_g_pairs, "prefill_flops_swa_layer": 4 * H * D * pre_s_pairs,
+            "prefill_flops_global_layer": 4 * H * Dg * pre_g_pairs, "prefill_flops_swa_layer": 4 * H * D * pre_s_pairs,
         }
 
     def launch(self, i=0, kernel_mask=0):
@@ -385,13 +393,14 @@ class MixedStep(Workload):
         if not self.plans:
             for swa in (True, False):
                 k, v, W = (self.ks, self.vs, self.W_swa) if swa else (self.kg, self.vg, self.W_global)
+                qp, qd, op, od = (self.qp, self.qd, self.op, self.od) if swa else (self.qpg, self.qdg, self.opg, self.odg)
                 if self.one_launch:
-                    self.plans[swa] = (fa2.plan_flash_attention(self.qp, k, v, self.op, self.tds, self.phase, W, fa2.PHASE_PREFILL,
-                                                                scale=SCALE, workspace=self.ws, decode_q=self.qd, decode_o=self.od),)
+                    self.plans[swa] = (fa2.plan_flash_attention(qp, k, v, op, self.tds, self.phase, W, fa2.PHASE_PREFILL,
+                                                                scale=SCALE, workspace=self.ws, decode_q=qd, decode_o=od),)
                     continue
                 self.plans[swa] = (
-                    fa2.plan_flash_attention(self.qp, k, v, self.op, self.tds, self.phase, W, fa2.PHASE_PREFILL, scale=SCALE),
-                    fa2.plan_flash_attention(self.qd, k, v, self.od, self.tds, self.phase, W, fa2.PHASE_DECODE, scale=SCALE,
+                    fa2.plan_flash_attention(qp, k, v, op, self.tds, self.phase, W, fa2.PHASE_PREFILL, scale=SCALE),
+                    fa2.plan_flash_attention(qd, k, v, od, self.tds, self.phase, W, fa2.PHASE_DECODE, scale=SCALE,
                                              workspace=self.ws),
                 )
         for layer in range(self.layers):
@@ -454,6 +463,9 @@ WORKLOADS = {
     "prefill_causal_8192_bf16": lambda dev: Prefill(dev, 8192, bf16=True),
     "mixed_step": lambda dev: MixedStep(dev),
     "mixed_step_two_launches": lambda dev: MixedStep(dev, one_launch=False),
+    # the same step with Gemma-4's layer shapes: head dimension 256 on sliding-window layers, 512 on global ones
+    "mixed_step_global_d512": lambda dev: MixedStep(dev, global_dim=512),
+    "mixed_step_global_d512_two_launches": lambda dev: MixedStep(dev, global_dim=512, one_launch=False),
     "rope_append": lambda dev: RopeAppend(dev),
 }
 

@@ -282,7 +282,8 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
 // half gets what lets its stream run at full rate, the chunk the rest.
 namespace {
 constexpr int kMixedCus = 256;
-constexpr int kMixedDecodeBlocks = 80;  // decode workgroups (four one-wave workers each) asked for by default
+constexpr int kMixedDecodeBlocks = 80;  // decode workgroups asked for by default (four one-wave workers each; at head
+                                        // dimension 512 one four-wave worker each)
 
 struct MixedShape {
     int split_slots;     // (active slot, key split) pairs of the prefill half; <= 1 = unsplit
@@ -291,18 +292,21 @@ struct MixedShape {
     uint64_t pf_bytes, dec_bytes;
 };
 
-// B, H, G, D, KV_CTX, W, window_sizes are shared; tq_pf / tq_dec are the query tokens per slot of the two halves.
-MixedShape mixed_shape(int B, int H, int G, int D, int tq_pf, int tq_dec, bool pair_path, int num_workers, bool with_ws) {
+// B, H, G, D, KV_CTX, W, window_sizes are shared; tq_pf / tq_dec are the query tokens per slot of the two halves;
+// pf_rows = query rows of a prefill workgroup.
+MixedShape mixed_shape(int B, int H, int G, int D, int tq_pf, int tq_dec, bool pair_path, int num_workers, bool with_ws,
+                       int pf_rows = 128) {
     MixedShape m{};
-    const int R = H / G, tokb = 128 / R;
+    const int R = H / G, tokb = pf_rows / R;
+    const int wpb = D == 512 ? 1 : 4;                      // decode workers per workgroup
     const int per_slot = ((tq_pf + tokb - 1) / tokb) * G;  // prefill workgroups one slot brings unsplit
-    int nd = pair_path ? B * G : (num_workers > 0 ? (num_workers + 3) / 4 : kMixedDecodeBlocks);
-    if (!with_ws && !pair_path) nd = (B * G + 3) / 4;  // one worker per pair
+    int nd = pair_path ? B * G : (num_workers > 0 ? (num_workers + wpb - 1) / wpb : kMixedDecodeBlocks);
+    if (!with_ws && !pair_path) nd = (B * G + wpb - 1) / wpb;  // one worker per pair
     int slots = with_ws ? (kMixedCus - nd) / per_slot : 1;
     slots = slots < 1 ? 1 : (slots > kPrefillMaxSplitSlots ? kPrefillMaxSplitSlots : slots);
     if (!pair_path && with_ws && num_workers <= 0 && slots * per_slot + nd < kMixedCus) nd = kMixedCus - slots * per_slot;
     m.split_slots = slots >= 2 ? slots : 0;
-    m.nw = (pair_path || !with_ws) ? 0 : nd * 4;
+    m.nw = (pair_path || !with_ws) ? 0 : nd * wpb;
     m.plan.nd_blocks = nd;
     m.plan.pair_path = pair_path ? 1 : 0;
     m.pf_bytes = (uint64_t)m.split_slots * H * tq_pf * (uint64_t)(D + 2) * sizeof(float);
@@ -336,15 +340,17 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
     if ((int64_t)pp.R * pp.Tq <= kMaxDecodeRows || (int64_t)pd.R * pd.Tq > kMaxDecodeRows)
         return fail(G4B_ERR_INVALID_ARGUMENT, "mixed launch: the first block must be prefill-shaped ((H/G)*Tq > %d), the second "
                     "decode-shaped", kMaxDecodeRows);
-    if (a->D != 256) return fail(G4B_ERR_UNSUPPORTED, "mixed launch is built for head_dim 256 (got %d)", a->D);
-    if (128 % pp.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide 128 for prefill-shaped launches", pp.R);
+    if (a->D != 256 && a->D != 512) return fail(G4B_ERR_UNSUPPORTED, "mixed launch is built for head_dim 256 and 512 (got %d)", a->D);
+    // a split query halves the rows of a head-dimension-512 prefill workgroup
+    const int pf_rows = prefill_rows_per_workgroup(a->D) / ((a->D == 512 && pp.q_split) ? 2 : 1);
+    if (pf_rows % pp.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide %d for this prefill shape", pp.R, pf_rows);
     if (pp.q_split != pd.q_split)
         return fail(G4B_ERR_UNSUPPORTED, "mixed launch: both halves must take the same query precision path (same q dtype and use_fp32_dot)");
     if (a->kernel_mask != d->kernel_mask) return fail(G4B_ERR_INVALID_ARGUMENT, "mixed launch: kernel_mask must agree");
 
     const bool pair = g4b::decode_pair_path(pd, a->D);
     const bool with_ws = a->workspace != nullptr;
-    const MixedShape m = mixed_shape(a->B, a->H, a->G, a->D, a->Tq, d->Tq, pair, d->num_workers, with_ws);
+    const MixedShape m = mixed_shape(a->B, a->H, a->G, a->D, a->Tq, d->Tq, pair, d->num_workers, with_ws, pf_rows);
     if (with_ws) {
         // one workspace, passed with the prefill block: the chunk's partials first, the decode partials after them
         const uint64_t pf_span = (m.pf_bytes + 255) & ~(uint64_t)255;
@@ -364,13 +370,14 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
         }
     }
     g4b::MixedPlan mp = m.plan;
-    mp.npx = (g4b::prefill_grid(pp) + 7) / 8;
+    mp.npx = (g4b::prefill_grid(pp, pf_rows, a->D != 512) + 7) / 8;
     mp.combine_pf = g4b::prefill_combine_grid(pp);
     mp.combine_dec = (pair || !m.nw) ? 0 : a->B * a->G * pd.R * pd.Tq;
     if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
-    const hipError_t e = a->kv_dtype == G4B_DT_F16
-                             ? g4b::launch_attn_mixed_f16(pp, pd, mp, a->D, static_cast<hipStream_t>(stream))
-                             : g4b::launch_attn_mixed_bf16(pp, pd, mp, a->D, static_cast<hipStream_t>(stream));
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (a->D == 512) e = a->kv_dtype == G4B_DT_F16 ? g4b::launch_attn_mixed_d512_f16(pp, pd, mp, st) : g4b::launch_attn_mixed_d512_bf16(pp, pd, mp, st);
+    else e = a->kv_dtype == G4B_DT_F16 ? g4b::launch_attn_mixed_f16(pp, pd, mp, st) : g4b::launch_attn_mixed_bf16(pp, pd, mp, st);
     profile_disarm();
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "mixed attention launch failed: %s", hipGetErrorString(e));
     return G4B_OK;

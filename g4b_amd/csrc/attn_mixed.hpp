@@ -10,9 +10,14 @@
 // (slot, kv head) pair of the short-window variant).  Both kinds occupy a compute unit alone (registers, LDS), so
 // the hardware places prefill and decode workgroups side by side on different units and the chunk's matrix work runs
 // under the stream's memory time.  A second launch merges the split partials of both halves.
+//
+// Head dimension 512: the prefill workgroups run the body of the 512 kernel, and a decode workgroup is ONE worker
+// whose four waves own 128 columns each (the streaming kernel's column split, which adds the waves' partial dot
+// products through LDS once per tile).
 #pragma once
 #include "attn_decode.hpp"
 #include "attn_prefill.hpp"
+#include "attn_prefill_wide.hpp"
 #include "launch.hpp"
 
 namespace g4b {
@@ -25,15 +30,20 @@ __global__ __launch_bounds__(256) void attn_mixed_kernel(const AttnParams pp, co
     const int ndx = (mp.nd_blocks + 7) >> 3;
     if (j >= ndx) {
         // the prefill grid is sized for every slot being in the prefill phase; the surplus leaves at once
-        prefill_body<D, T, QS>(pp, (j - ndx) * 8 + x, smem, sh_scan);
+        if constexpr (D == 512) prefill_wide_body<T, QS>(pp, (j - ndx) * 8 + x, smem, sh_scan);
+        else prefill_body<D, T, QS>(pp, (j - ndx) * 8 + x, smem, sh_scan);
         return;
     }
     const int d = j * 8 + x;
     if (d >= mp.nd_blocks) return;
-    if (mp.pair_path) {
-        decode_pair_body<D, CL, T, QS>(pd, d, reinterpret_cast<float*>(smem));
+    if constexpr (D == 512) {
+        decode_worker_body<D, CL, T, 4, QS>(pd, d, reinterpret_cast<float*>(smem));
     } else {
-        decode_worker_body<D, CL, T, 1, QS>(pd, d * 4 + (int)(threadIdx.x >> 6), nullptr);
+        if (mp.pair_path) {
+            decode_pair_body<D, CL, T, QS>(pd, d, reinterpret_cast<float*>(smem));
+        } else {
+            decode_worker_body<D, CL, T, 1, QS>(pd, d * 4 + (int)(threadIdx.x >> 6), nullptr);
+        }
     }
 }
 
@@ -51,7 +61,8 @@ __global__ __launch_bounds__(256) void attn_mixed_combine(const AttnParams pp, c
 
 template <int D, int CL, class T, bool QS>
 static hipError_t launch_mixed_t(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream) {
-    constexpr int smem_pf = 4 * PfSmem<D>::TILE, smem_pair = dec_pair_smem<D>();
+    constexpr int smem_pf = D == 512 ? PW_SMEM : 4 * PfSmem<D>::TILE;
+    constexpr int smem_pair = D == 512 ? 2 * 4 * 8 * 64 * (int)sizeof(float) : dec_pair_smem<D>();  // 512: the workers' exchange buffers
     constexpr int smem = smem_pf > smem_pair ? smem_pf : smem_pair;
     static uint64_t attr_done = 0;
     hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_mixed_kernel<D, CL, T, QS>), smem, attr_done);
@@ -65,18 +76,17 @@ static hipError_t launch_mixed_t(const AttnParams& pp, const AttnParams& pd, con
     return hipGetLastError();
 }
 
-template <class T>
-static hipError_t launch_mixed_dtype(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, int D, hipStream_t stream) {
+template <int D, class T>
+static hipError_t launch_mixed_dtype(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream) {
     const int rows = pd.R * pd.Tq;
-    if (D != 256) return hipErrorInvalidValue;
     if (pp.q_split) {
-        if (rows <= 4) return launch_mixed_t<256, 4, T, true>(pp, pd, mp, stream);
-        if (rows <= 8) return launch_mixed_t<256, 2, T, true>(pp, pd, mp, stream);
-        return launch_mixed_t<256, 1, T, true>(pp, pd, mp, stream);
+        if (rows <= 4) return launch_mixed_t<D, 4, T, true>(pp, pd, mp, stream);
+        if (rows <= 8) return launch_mixed_t<D, 2, T, true>(pp, pd, mp, stream);
+        return launch_mixed_t<D, 1, T, true>(pp, pd, mp, stream);
     }
-    if (rows <= 4) return launch_mixed_t<256, 4, T, false>(pp, pd, mp, stream);
-    if (rows <= 8) return launch_mixed_t<256, 2, T, false>(pp, pd, mp, stream);
-    return launch_mixed_t<256, 1, T, false>(pp, pd, mp, stream);
+    if (rows <= 4) return launch_mixed_t<D, 4, T, false>(pp, pd, mp, stream);
+    if (rows <= 8) return launch_mixed_t<D, 2, T, false>(pp, pd, mp, stream);
+    return launch_mixed_t<D, 1, T, false>(pp, pd, mp, stream);
 }
 
 }  // namespace g4b

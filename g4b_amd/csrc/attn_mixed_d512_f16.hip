@@ -1,0 +1,8 @@
+// Mixed prefill + decode launch, f16 caches, head dimension 512 (attn_mixed.hpp).
+#include "attn_mixed.hpp"
+
+namespace g4b {
+hipError_t launch_attn_mixed_d512_f16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream) {
+    return launch_mixed_dtype<512, F16>(pp, pd, mp, stream);
+}
+}  // namespace g4b

@@ -62,8 +62,12 @@ struct MixedPlan {
     int combine_pf;   // merge workgroups of the prefill half
     int combine_dec;  // merge workgroups of the decode half
 };
-hipError_t launch_attn_mixed_f16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, int D, hipStream_t stream);
-hipError_t launch_attn_mixed_bf16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, int D, hipStream_t stream);
+// head dimension 256
+hipError_t launch_attn_mixed_f16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream);
+hipError_t launch_attn_mixed_bf16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream);
+// head dimension 512
+hipError_t launch_attn_mixed_d512_f16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream);
+hipError_t launch_attn_mixed_d512_bf16(const AttnParams& pp, const AttnParams& pd, const MixedPlan& mp, hipStream_t stream);
 
 struct KvAppendParams {
     const void* x;

@@ -254,7 +254,7 @@ def flash_attention(
       ``phase``) also computes ``decode_o`` from ``decode_q`` for the slots in ``decode_phase``, in the same grid:
       the chunk's workgroups and the decode stream's run on different compute units at the same time.  Same results
       as the two calls.  ``workspace`` must then be a tensor of :func:`mixed_workspace_bytes` bytes (or absent: no
-      half splits its keys).  Head dimension 256.
+      half splits its keys).  Head dimensions 256 and 512.
 
     Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
     ignore (``g4b/models/gemma4e.py:593-607``).

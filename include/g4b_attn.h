@@ -137,7 +137,7 @@ int32_t g4b_attn_default_workers(void);
  * ((H/G)*Tq <= 16); they must name the same caches, time_dim_sizes, user_phase, window_sizes, B, H, G, D, KV_CTX, cache
  * dtype and ctx_window_size and differ in q, o, Tq, strides and phase.  Results are those of the two calls.  The
  * workgroups of the two halves are dealt to different compute units, so the chunk's matrix work runs under the decode
- * stream's memory time.  Head dimension 256.
+ * stream's memory time.  Head dimensions 256 and 512.
  *   workspace     one buffer for both halves, passed in `prefill->workspace` (`decode->workspace` is ignored), at
  *                 least g4b_attn_mixed_workspace_bytes(...) bytes; NULL = neither half splits keys.
  *   num_workers   `decode->num_workers`: 0 = the library's share-out of the chip between the halves.

@@ -26,7 +26,7 @@ def fa(gpu_device):
     return fa2
 
 
-def make_batch(B, t, kv_ctx, seed, dtype=torch.float16, q_dtype=None):
+def make_batch(B, t, kv_ctx, seed, dtype=torch.float16, q_dtype=None, D=D):
     gen = torch.Generator(device="cpu").manual_seed(seed)
     q_dtype = q_dtype or dtype
     qp = torch.randn(B, H, t, D, generator=gen).to(q_dtype).cuda()
@@ -65,14 +65,15 @@ def check_both_halves(fa, qp, qd, k, v, tds, phase, W, scale, ws, tol=None, **kw
 
 @pytest.mark.parametrize("layer", ["global", "sliding_window"])
 @pytest.mark.parametrize("with_workspace", [True, False], ids=["split", "unsplit"])
-def test_mixed_step_matches_the_oracle(fa, layer, with_workspace):
-    print(f"mixed {layer} workspace={with_workspace}", flush=True)
+@pytest.mark.parametrize("D", [256, 512])
+def test_mixed_step_matches_the_oracle(fa, layer, with_workspace, D):
+    print(f"mixed {layer} workspace={with_workspace} D={D}", flush=True)
     B, t = 9, 128
     if layer == "global":
         W = kv_ctx = 3000 + t - 1
     else:
         W, kv_ctx = 512, 512 + t - 1
-    qp, qd, k, v = make_batch(B, t, kv_ctx, seed=31)
+    qp, qd, k, v = make_batch(B, t, kv_ctx, seed=31, D=D)
     # slots 0-5 decode (lengths 1 .. beyond the ring, one empty), 6 a chunk on a long context, 7 unallocated, 8 a
     # chunk at the start of its sequence
     tds = [1, 77, 2900, 1500, 0, 2999 if layer == "global" else kv_ctx + 40, 2000 + t, 9, t]
@@ -104,11 +105,12 @@ def test_mixed_step_equals_the_two_separate_launches_closely(fa):
     assert (od.float() - od2.float()).abs().max().item() <= 4e-3
 
 
-def test_mixed_step_fp32_queries_and_per_slot_windows(fa):
+@pytest.mark.parametrize("D", [256, 512])
+def test_mixed_step_fp32_queries_and_per_slot_windows(fa, D):
     """Engine-style fp32 q with use_fp32_dot on a bf16 cache (split-query kernels), and per-slot window sizes (which
     force the streaming workers even for short windows)."""
     B, t, kv_ctx = 4, 96, 1500
-    qp, qd, k, v = make_batch(B, t, kv_ctx, seed=33, dtype=torch.bfloat16, q_dtype=torch.float32)
+    qp, qd, k, v = make_batch(B, t, kv_ctx, seed=33, dtype=torch.bfloat16, q_dtype=torch.float32, D=D)
     tds, phase = [1400, 700 + t, 90, 1500], [2, 1, 2, 2]
     win = [512, kv_ctx, kv_ctx, 64]
     n = fa.mixed_workspace_bytes(B, H, G, t, 1, D, kv_ctx, kv_ctx, True)

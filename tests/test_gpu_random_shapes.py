@@ -45,8 +45,9 @@ def draw_case(rng):
     engine = rng.random() < 0.5
     split = rng.random() < 0.5
     scale = float(rng.choice([1.0, 1 / 16, 0.3]))
+    fp32_dot = rng.random() < 0.5  # drawn last: the cases keep the parameters they had before this switch existed
     return dict(D=D, H=H, G=G, Tq=Tq, kv_ctx=kv_ctx, W=W, B=B, phase_id=phase_id, phase=phase, tds=tds, stage=stage, qwin=qwin,
-                win=win, bf16=bf16, q_f32=q_f32, engine=engine, split=split, scale=scale)
+                win=win, bf16=bf16, q_f32=q_f32, engine=engine, split=split, scale=scale, fp32_dot=fp32_dot)
 
 
 @pytest.mark.parametrize("n", range(N_CASES))
@@ -69,8 +70,10 @@ def test_random_launch(gpu_device, n):
     k = torch.randn(B, G, c["kv_ctx"], D, generator=gen).to(cdt).cuda()
     v = torch.randn(B, G, c["kv_ctx"], D, generator=gen).to(cdt).cuda()
     kw = dict(stage=c["stage"], scale=c["scale"], query_window=c["qwin"])
-    # the kernels feed the MFMA with q rounded to the cache's 16-bit type
-    ref = oracle(q.to(cdt), k, v, c["tds"], c["phase"], c["W"], c["phase_id"], window_sizes=c["win"], **kw)
+    # use_fp32_dot=False: the kernels feed the MFMA with q rounded to the cache's 16-bit type (fa2.py:88);
+    # use_fp32_dot=True: with the query as a hi + lo pair of operands, i.e. the oracle on the query as it is
+    ref = oracle(q if c["fp32_dot"] else q.to(cdt), k, v, c["tds"], c["phase"], c["W"], c["phase_id"], window_sizes=c["win"], **kw)
+    kw["use_fp32_dot"] = c["fp32_dot"]
     if c["win"] is not None:
         kw["window_sizes"] = i32(c["win"])
     if c["split"]:
@@ -180,3 +183,77 @@ def test_random_kv_append_is_bit_exact(gpu_device, n):
         rows = (torch.arange(t) + offs[b]) % T
         exp[b][:, rows.cuda(), :] = x[b].to(cdt)
     assert torch.equal(cache, exp), dict(D=D, G=G, B=B, T=T, t=t, offs=offs, phase=phase if use_phase else None)
+
+
+N_MIXED_CASES = 60
+
+
+@pytest.mark.parametrize("n", range(N_MIXED_CASES))
+def test_random_mixed_launch(gpu_device, n):
+    """Prefill-phase and decode-phase slots in one launch (decode_q= / decode_o=): random group sizes, chunk lengths,
+    rings, windows, phases (including slots of neither phase), lengths, dtypes, with and without a workspace, against
+    the oracle run once per phase."""
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(9000 + n)
+    D = int(rng.choice([256, 512]))
+    R = int(rng.choice([1, 2, 4, 8, 16]))
+    G = int(rng.choice([1, 2, 3]))
+    H = R * G
+    t = int(rng.choice([17, 33, 64, 100, 130]))
+    td = int(rng.choice([1, 1, 1, 2, 3]))
+    if R * td > 16:
+        td = 1
+    kv_ctx = int(rng.integers(t + 8, 400))
+    W = int(rng.integers(t, kv_ctx + 1)) if rng.random() < 0.7 else kv_ctx
+    B = int(rng.integers(2, 8))
+    phase = [int(rng.choice([1, 2, 2, 2, 0])) for _ in range(B)]
+    tds = []
+    for b in range(B):
+        lo = t if phase[b] == 1 else td
+        kind = rng.integers(0, 4)
+        if kind == 0:
+            tds.append(lo if phase[b] == 1 else int(rng.choice([0, td])))
+        elif kind == 1:
+            tds.append(int(rng.integers(lo, max(lo, W) + 1)))
+        else:
+            tds.append(int(rng.integers(W, 4 * kv_ctx)))
+    win = [int(rng.integers(t, W + 1)) for _ in range(B)] if rng.random() < 0.25 else None
+    bf16, q_f32, fp32_dot = rng.random() < 0.25, rng.random() < 0.4, rng.random() < 0.5
+    with_ws = rng.random() < 0.7
+    scale = float(rng.choice([1.0, 1 / 16, 0.3]))
+    print(dict(D=D, H=H, G=G, t=t, td=td, kv_ctx=kv_ctx, W=W, B=B, phase=phase, tds=tds, win=win, bf16=bf16, q_f32=q_f32,
+               fp32_dot=fp32_dot, with_ws=with_ws, scale=scale), flush=True)
+    cdt = torch.bfloat16 if bf16 else torch.float16
+    qdt = torch.float32 if q_f32 else cdt
+    gen = torch.Generator().manual_seed(9500 + n)
+    qp = torch.randn(B, t, H, D, generator=gen).to(qdt).cuda().permute(0, 2, 1, 3)
+    qd = torch.randn(B, td, H, D, generator=gen).to(qdt).cuda().permute(0, 2, 1, 3)
+    op = torch.full((B, t, H, D), 777.0, dtype=qdt, device="cuda").permute(0, 2, 1, 3)
+    od = torch.full((B, td, H, D), 777.0, dtype=qdt, device="cuda").permute(0, 2, 1, 3)
+    k = torch.randn(B, G, kv_ctx, D, generator=gen).to(cdt).cuda()
+    v = torch.randn(B, G, kv_ctx, D, generator=gen).to(cdt).cuda()
+    kw = dict(scale=scale, use_fp32_dot=fp32_dot)
+    if win is not None:
+        kw["window_sizes"] = i32(win)
+    if with_ws:
+        nbytes = fa2.mixed_workspace_bytes(B, H, G, t, td, D, kv_ctx, W, win is not None)
+        kw["workspace"] = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    fa2.flash_attention(qp, k, v, op, i32(tds), u8(phase), W, 1, decode_q=qd, decode_o=od, **kw)
+    torch.cuda.synchronize()
+    rq = (lambda x: x) if fp32_dot else (lambda x: x.to(cdt))
+    ref_p = oracle(rq(qp), k, v, tds, phase, W, 1, scale=scale, window_sizes=win)
+    ref_d = oracle(rq(qd), k, v, tds, phase, W, 2, scale=scale, window_sizes=win)
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if bf16 else {}
+    sentinel = torch.tensor(777.0, dtype=qdt).float().item()
+    gp, gd = op.float().cpu().numpy(), od.float().cpu().numpy()
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(gp[b], ref_p[b], what=f"mixed case {n} chunk slot {b}", **tol)
+            assert (gd[b] == sentinel).all()
+        elif phase[b] == 2:
+            if tds[b] >= td:  # a decode slot shorter than its query block is the caller's to avoid (scheduler.py:167-172)
+                assert_close(gd[b], ref_d[b], what=f"mixed case {n} decode slot {b}", **tol)
+            assert (gp[b] == sentinel).all()
+        else:
+            assert (gp[b] == sentinel).all() and (gd[b] == sentinel).all(), f"mixed case {n}: idle slot {b} was written"

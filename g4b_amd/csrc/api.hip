@@ -282,8 +282,11 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
 // half gets what lets its stream run at full rate, the chunk the rest.
 namespace {
 constexpr int kMixedCus = 256;
-constexpr int kMixedDecodeBlocks = 80;  // decode workgroups asked for by default (four one-wave workers each; at head
-                                        // dimension 512 one four-wave worker each)
+// Decode workgroups asked for by default: four one-wave workers each at head dimension 256 (the stream reaches its
+// rate with 320..384 workers); one four-wave worker each at 512, whose waves keep half as many bytes in flight and
+// need more of the chip (measured on the benchmark's global layers: 96 workgroups 381 us, 128 327 us, 160 380 us).
+constexpr int kMixedDecodeBlocks = 80;
+constexpr int kMixedDecodeBlocksWide = 112;
 
 struct MixedShape {
     int split_slots;     // (active slot, key split) pairs of the prefill half; <= 1 = unsplit
@@ -300,7 +303,7 @@ MixedShape mixed_shape(int B, int H, int G, int D, int tq_pf, int tq_dec, bool p
     const int R = H / G, tokb = pf_rows / R;
     const int wpb = D == 512 ? 1 : 4;                      // decode workers per workgroup
     const int per_slot = ((tq_pf + tokb - 1) / tokb) * G;  // prefill workgroups one slot brings unsplit
-    int nd = pair_path ? B * G : (num_workers > 0 ? (num_workers + wpb - 1) / wpb : kMixedDecodeBlocks);
+    int nd = pair_path ? B * G : (num_workers > 0 ? (num_workers + wpb - 1) / wpb : (D == 512 ? kMixedDecodeBlocksWide : kMixedDecodeBlocks));
     if (!with_ws && !pair_path) nd = (B * G + wpb - 1) / wpb;  // one worker per pair
     int slots = with_ws ? (kMixedCus - nd) / per_slot : 1;
     slots = slots < 1 ? 1 : (slots > kPrefillMaxSplitSlots ? kPrefillMaxSplitSlots : slots);

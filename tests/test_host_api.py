@@ -209,3 +209,51 @@ def test_pipelined_kernels_keep_foreign_memory_traffic_out_of_their_wait_regions
     # head dims 128, 256 and 512, fp16 and bf16 caches, each with the query rounded or split into two operands
     assert len(seen) == 12, seen
     assert all(n >= 48 for n in seen.values()), seen
+
+
+def test_mixed_launch_is_validated_before_launching(native):
+    """g4b_attn_forward_mixed checks both argument blocks and their agreement on the host (no GPU needed)."""
+    from g4b_amd.kernels.fa2 import PHASE_DECODE, PHASE_PREFILL, flash_attention, mixed_workspace_bytes
+
+    lib = native.load()
+    assert lib.g4b_attn_forward_mixed(None, None, None) == native.G4B_ERR_INVALID_ARGUMENT
+    B, H, G, D, T, t = 2, 8, 2, 256, 600, 64
+    qp, qd = torch.zeros(B, H, t, D, dtype=torch.float16), torch.zeros(B, H, 1, D, dtype=torch.float16)
+    k = torch.zeros(B, G, T, D, dtype=torch.float16)
+    tds, ph = torch.zeros(B, dtype=torch.int32), torch.zeros(B, dtype=torch.uint8)
+    with pytest.raises(ValueError, match="go together"):
+        flash_attention(qp, k, k, qp.clone(), tds, ph, T, PHASE_PREFILL, decode_q=qd)
+    with pytest.raises(ValueError, match="different phases"):
+        flash_attention(qp, k, k, qp.clone(), tds, ph, T, PHASE_DECODE, decode_q=qd, decode_o=qd.clone())
+    with pytest.raises(ValueError, match="prefill-shaped"):
+        flash_attention(qd, k, k, qd.clone(), tds, ph, T, PHASE_PREFILL, decode_q=qd, decode_o=qd.clone())
+    with pytest.raises(ValueError, match="partial_o"):
+        flash_attention(qp, k, k, qp.clone(), tds, ph, T, PHASE_PREFILL, torch.zeros(4, B, H, t, D), torch.zeros(4, B, H, t),
+                        torch.zeros(4, B, H, t), decode_q=qd, decode_o=qd.clone())
+    with pytest.raises(ValueError, match="workspace holds"):
+        flash_attention(qp, k, k, qp.clone(), tds, ph, T, PHASE_PREFILL, decode_q=qd, decode_o=qd.clone(),
+                        workspace=torch.zeros(64, dtype=torch.uint8))
+    q128, k128 = torch.zeros(B, H, t, 128, dtype=torch.float16), torch.zeros(B, G, T, 128, dtype=torch.float16)
+    with pytest.raises(NotImplementedError, match="head_dim"):
+        flash_attention(q128, k128, k128, q128.clone(), tds, ph, T, PHASE_PREFILL, decode_q=torch.zeros(B, H, 1, 128, dtype=torch.float16),
+                        decode_o=torch.zeros(B, H, 1, 128, dtype=torch.float16))
+    # sizing: the chunk's partials ((slot, split) pairs x H x t x (D + 2) floats, rounded up to 256 bytes) followed by the
+    # decode partials ((workers + B*G) x rows x (D + 2) floats).  64-token chunks bring 2 tiles x 2 kv heads = 4 workgroups
+    # per slot; the default share-out leaves 256 - 80 = 176 units to the chunk -> 44 pairs, and the decode half gets the
+    # remaining 80 workgroups of four workers.
+    n = mixed_workspace_bytes(B, H, G, t, 1, D, T, T)
+    assert n == 44 * H * t * (D + 2) * 4 + (320 + B * G) * 4 * (D + 2) * 4
+    # a short window takes the one-workgroup-per-pair decode path: no decode partials, 256 - B*G units for the chunk
+    n_swa = mixed_workspace_bytes(B, H, G, t, 1, D, 512 + t - 1, 512)
+    assert n_swa == 63 * H * t * (D + 2) * 4
+    assert mixed_workspace_bytes(B, H, G, t, 1, D, 512 + t - 1, 512, True) == n  # per-slot windows: streaming workers again
+
+
+def test_static_scratch_entry_point_checks_its_arguments(native):
+    lib = native.load()
+    assert lib.g4b_static_scratch_bytes() == 68 << 20
+    assert lib.g4b_attn_forward_static_scratch(None, None) == native.G4B_ERR_INVALID_ARGUMENT
+    a = native.AttnArgs()
+    a.workspace = 4096
+    assert lib.g4b_attn_forward_static_scratch(ctypes.byref(a), None) == native.G4B_ERR_INVALID_ARGUMENT
+    assert "workspace must be NULL" in native.last_error()

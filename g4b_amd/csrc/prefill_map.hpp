@@ -59,12 +59,16 @@ inline int prefill_grid(const AttnParams& p, int bm = PF_BM, bool paired = true)
     const int nq = (p.Tq + tokb - 1) / tokb;
     const int slots = p.part_o ? p.split_slots : 1;
     int blocks = 0;
-    for (int n = 1; n <= p.B; ++n) {
+    // keys are only split while 2 * n <= slots and the XCD-sharing map (up to 8 heads) rounds its grid up; beyond both
+    // the grid grows with n, so n = B is the largest
+    const int n_small = slots / 2 + 1 > 8 ? slots / 2 + 1 : 8;
+    for (int n = 1; n <= n_small && n <= p.B; ++n) {
         const int ns = prefill_splits(slots, n);
         const int g = pf_map(n * p.G * ns, paired ? pf_ranks(ns, nq) : nq).grid;
         blocks = g > blocks ? g : blocks;
     }
-    return blocks;
+    const int g_all = pf_map(p.B * p.G * prefill_splits(slots, p.B), paired ? pf_ranks(prefill_splits(slots, p.B), nq) : nq).grid;
+    return g_all > blocks ? g_all : blocks;
 }
 
 }  // namespace g4b

@@ -5,7 +5,8 @@
  *
  * Conventions
  *   - Every pointer is a device pointer owned by the caller; the library never allocates,
- *     frees or synchronises.  Work is enqueued on `stream` (a hipStream_t passed as void*;
+ *     frees or synchronises (the scratch of g4b_attn_forward_static_scratch is an array in the
+ *     library's device image, not an allocation).  Work is enqueued on `stream` (a hipStream_t passed as void*;
  *     NULL = the default stream) and is legal inside stream capture.
  *   - Strides are in ELEMENTS, as in the reference's launch adapter (g4b/kernels/utils.py:87-127).
  *   - Entry points return G4B_OK (0) or a negative g4b_status.  Arguments are validated on the

@@ -324,7 +324,14 @@ uint64_t g4b_attn_mixed_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t
     const int W = ctx_window_size < KV_CTX ? ctx_window_size : KV_CTX;
     const bool pair = D <= 256 && !has_window_sizes && W <= g4b::DEC_PAIR_MAX_KEYS;
     const MixedShape m = mixed_shape(B, H, G, D, Tq_prefill, Tq_decode, pair, num_workers, true);
-    return ((m.pf_bytes + 255) & ~(uint64_t)255) + m.dec_bytes;
+    uint64_t need = ((m.pf_bytes + 255) & ~(uint64_t)255) + m.dec_bytes;
+    if (D == 512 && 64 % (H / G) == 0) {
+        // a split query (fp32 q with use_fp32_dot) halves the rows of a prefill workgroup, which can move the share-out
+        const MixedShape h = mixed_shape(B, H, G, D, Tq_prefill, Tq_decode, pair, num_workers, true, 64);
+        const uint64_t need_h = ((h.pf_bytes + 255) & ~(uint64_t)255) + h.dec_bytes;
+        need = need_h > need ? need_h : need;
+    }
+    return need;
 }
 
 int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* decode, void* stream) {

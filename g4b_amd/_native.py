@@ -14,7 +14,7 @@ G4B_ERR_WORKSPACE = -3
 G4B_ERR_LAUNCH = -4
 
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class AttnArgs(C.Structure):
@@ -51,6 +51,7 @@ class AttnArgs(C.Structure):
         ("num_workers", C.c_int32),
         ("kernel_mask", C.c_int32),
         ("use_fp32_dot", C.c_int32),
+        ("on_band_block", C.c_int32),
         ("scale", C.c_float),
     ]
 

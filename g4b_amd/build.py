@@ -24,7 +24,8 @@ LIB_PATH = PKG_DIR / "libg4b_attn.so"
 ARCH = "gfx950"
 
 SOURCES = ["api.hip", "attn_decode.hip", "attn_prefill.hip", "attn_prefill_wide.hip", "attn_mixed_f16.hip",
-           "attn_mixed_bf16.hip", "attn_mixed_d512_f16.hip", "attn_mixed_d512_bf16.hip", "cache_ops.hip", "rope.hip"]
+           "attn_mixed_bf16.hip", "attn_mixed_d512_f16.hip", "attn_mixed_d512_bf16.hip", "attn_generic.hip", "cache_ops.hip",
+           "rope.hip"]
 
 # packed-fp32 VALU forms are kept off: the compiler must not form v_pk_{add,mul,fma}_f32
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -149,10 +149,24 @@ int32_t g4b_attn_default_workers(void) { return kDefaultWorkers; }
 
 uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers) {
     if (B < 1 || H < 1 || G < 1 || Tq < 1 || D < 1 || H % G) return 0;
+    if (D != 128 && D != 256 && D != 512) return 0;  // the plain fp32 kernel never splits
     const int64_t rows = (int64_t)(H / G) * Tq;
     if (rows > kMaxDecodeRows) return prefill_workspace_bytes(H, G, Tq, D);
     const int nw = num_workers > 0 ? num_workers : default_workers(D);
     return decode_slots(B, G, nw) * (uint64_t)rows * (uint64_t)(D + 2) * sizeof(float);
+}
+
+// Shapes and types the tuned kernels are not built for go to the plain fp32 kernel (attn_generic.hip): an fp32 cache,
+// STAGE_ON_BAND alone, head dimensions other than 128 / 256 / 512, and prefill-shaped launches whose H/G does not
+// divide a workgroup's query rows.  It never uses a workspace.
+static bool takes_generic_path(const g4b_attn_args* a) {
+    if (a->kv_dtype == G4B_DT_F32 || a->stage == G4B_STAGE_ON_BAND) return true;
+    if (a->D != 128 && a->D != 256 && a->D != 512) return true;
+    const int R = a->H / a->G;
+    if ((int64_t)R * a->Tq <= kMaxDecodeRows) return false;
+    const bool q_wider = a->q_dtype == G4B_DT_F32 || (a->q_dtype == G4B_DT_F16 && a->kv_dtype == G4B_DT_BF16);
+    const int bm = prefill_rows_per_workgroup(a->D) / ((a->D == 512 && a->use_fp32_dot && q_wider) ? 2 : 1);
+    return bm % R != 0;
 }
 
 // Host-side validation of one argument block and its translation into kernel parameters (everything except the
@@ -163,20 +177,19 @@ static int fill_attn_params(const g4b_attn_args* a, g4b::AttnParams& p) {
         return fail(G4B_ERR_INVALID_ARGUMENT, "q, k_cache, v_cache, o, time_dim_sizes and user_phase must be non-NULL");
     if (!dtype_ok(a->q_dtype) || !dtype_ok(a->o_dtype))
         return fail(G4B_ERR_INVALID_ARGUMENT, "q/o dtype must be f16, bf16 or f32 (got %d, %d)", a->q_dtype, a->o_dtype);
-    if (a->kv_dtype != G4B_DT_F16 && a->kv_dtype != G4B_DT_BF16)
-        return fail(G4B_ERR_UNSUPPORTED, "KV cache dtype must be f16 or bf16 (got %d)", a->kv_dtype);
+    if (!dtype_ok(a->kv_dtype)) return fail(G4B_ERR_INVALID_ARGUMENT, "KV cache dtype must be f16, bf16 or f32 (got %d)", a->kv_dtype);
     if (a->B < 1 || a->H < 1 || a->G < 1 || a->Tq < 1 || a->D < 1 || a->KV_CTX < 1)
         return fail(G4B_ERR_INVALID_ARGUMENT, "B, H, G, Tq, D, KV_CTX must be positive");
     if (a->H % a->G) return fail(G4B_ERR_INVALID_ARGUMENT, "H (%d) must be a multiple of G (%d)", a->H, a->G);
-    if (a->D != 128 && a->D != 256 && a->D != 512)
-        return fail(G4B_ERR_UNSUPPORTED, "head_dim %d not built (128, 256 and 512 are)", a->D);
+    if (a->D % 8 || a->D > 1024)
+        return fail(G4B_ERR_UNSUPPORTED, "head_dim must be a multiple of 8 and at most 1024 (got %d)", a->D);
     if (a->B > 65535 || a->G > 65535) return fail(G4B_ERR_UNSUPPORTED, "B and G must be <= 65535");
     if (a->ctx_window_size < 1 || a->ctx_window_size > a->KV_CTX)
         return fail(G4B_ERR_INVALID_ARGUMENT, "ctx_window_size (%d) must be in [1, KV_CTX = %d]", a->ctx_window_size, a->KV_CTX);
-    if (a->stage == G4B_STAGE_ON_BAND)
-        return fail(G4B_ERR_UNSUPPORTED, "STAGE_ON_BAND alone depends on the reference's tile size and is not built");
-    if (a->stage != G4B_STAGE_FULL && a->stage != G4B_STAGE_CAUSAL)
-        return fail(G4B_ERR_INVALID_ARGUMENT, "stage must be STAGE_FULL (1) or STAGE_CAUSAL (3), got %d", a->stage);
+    if (a->stage != G4B_STAGE_FULL && a->stage != G4B_STAGE_CAUSAL && a->stage != G4B_STAGE_ON_BAND)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "stage must be STAGE_FULL (1), STAGE_ON_BAND (2) or STAGE_CAUSAL (3), got %d", a->stage);
+    if (a->stage == G4B_STAGE_ON_BAND && a->on_band_block < 1)
+        return fail(G4B_ERR_INVALID_ARGUMENT, "STAGE_ON_BAND alone needs on_band_block >= 1 (the reference's Q_BLOCKSIZE_T)");
     if (a->phase < 0 || a->phase > 255) return fail(G4B_ERR_INVALID_ARGUMENT, "phase must fit uint8");
     if (a->query_window < 0) return fail(G4B_ERR_INVALID_ARGUMENT, "query_window must be >= 0");
     if (!std::isfinite(a->scale) || !(a->scale > 0.f)) return fail(G4B_ERR_INVALID_ARGUMENT, "scale must be finite and positive");
@@ -190,8 +203,8 @@ static int fill_attn_params(const g4b_attn_args* a, g4b::AttnParams& p) {
     const int64_t slot_elems = (int64_t)a->G * a->KV_CTX * a->D;
     if (a->k_stride_b < slot_elems || a->v_stride_b < slot_elems || a->k_stride_b % 8 || a->v_stride_b % 8)
         return fail(G4B_ERR_INVALID_ARGUMENT, "cache slot stride must be >= G*KV_CTX*D and a multiple of 8 elements");
-    if ((int64_t)a->KV_CTX * a->D * 2 >= (int64_t)1 << 31)
-        return fail(G4B_ERR_UNSUPPORTED, "KV_CTX * D * 2 bytes must be below 2 GiB per (slot, kv head)");
+    if ((int64_t)a->KV_CTX * a->D * (a->kv_dtype == G4B_DT_F32 ? 4 : 2) >= (int64_t)1 << 31)
+        return fail(G4B_ERR_UNSUPPORTED, "one (slot, kv head) of the cache must stay below 2 GiB");
     if (a->num_workers < 0 || a->num_workers > (1 << 20)) return fail(G4B_ERR_INVALID_ARGUMENT, "num_workers out of range");
 
     p = g4b::AttnParams{};
@@ -236,7 +249,11 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     if (const int rc = fill_attn_params(a, p)) return rc;
     const int64_t rows = (int64_t)p.R * p.Tq;
     hipError_t e;
-    if (rows <= kMaxDecodeRows) {
+    if (takes_generic_path(a)) {
+        if ((int64_t)a->B * a->H * a->Tq > 0x7fffffffLL) return fail(G4B_ERR_UNSUPPORTED, "B * H * Tq must be below 2^31 on this path");
+        if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
+        e = g4b::launch_attn_generic(p, a->D, a->kv_dtype, a->on_band_block, static_cast<hipStream_t>(stream));
+    } else if (rows <= kMaxDecodeRows) {
         if (a->workspace) {
             const int nw = a->num_workers > 0 ? a->num_workers : default_workers(a->D);
             const uint64_t need = g4b_attn_workspace_bytes(a->B, a->H, a->G, a->Tq, a->D, nw);
@@ -253,10 +270,6 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
-        // a split query halves the rows of a head-dimension-512 workgroup
-        const int bm = prefill_rows_per_workgroup(a->D) / ((a->D == 512 && p.q_split) ? 2 : 1);
-        if (bm % p.R)
-            return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide %d for prefill-shaped launches with head_dim %d", p.R, bm, a->D);
         p.split_slots = 0;
         const uint64_t need = prefill_workspace_bytes(a->H, a->G, a->Tq, a->D);
         if (a->workspace && need) {
@@ -351,6 +364,8 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
         return fail(G4B_ERR_INVALID_ARGUMENT, "mixed launch: the first block must be prefill-shaped ((H/G)*Tq > %d), the second "
                     "decode-shaped", kMaxDecodeRows);
     if (a->D != 256 && a->D != 512) return fail(G4B_ERR_UNSUPPORTED, "mixed launch is built for head_dim 256 and 512 (got %d)", a->D);
+    if (a->kv_dtype == G4B_DT_F32 || a->stage == G4B_STAGE_ON_BAND || d->stage == G4B_STAGE_ON_BAND)
+        return fail(G4B_ERR_UNSUPPORTED, "mixed launch is built for f16 / bf16 caches and the causal and full stages");
     // a split query halves the rows of a head-dimension-512 prefill workgroup
     const int pf_rows = prefill_rows_per_workgroup(a->D) / ((a->D == 512 && pp.q_split) ? 2 : 1);
     if (pf_rows % pp.R) return fail(G4B_ERR_UNSUPPORTED, "H/G = %d must divide %d for this prefill shape", pp.R, pf_rows);
@@ -405,7 +420,8 @@ uint64_t g4b_static_scratch_bytes(void) { return kStaticScratchBytes; }
 int g4b_attn_forward_static_scratch(const g4b_attn_args* a, void* stream) {
     if (!a) return fail(G4B_ERR_INVALID_ARGUMENT, "args is NULL");
     if (a->workspace) return fail(G4B_ERR_INVALID_ARGUMENT, "g4b_attn_forward_static_scratch brings its own scratch: workspace must be NULL");
-    const uint64_t need = g4b_attn_workspace_bytes(a->B, a->H, a->G, a->Tq, a->D, a->num_workers);
+    const bool shape_ok = a->B >= 1 && a->H >= 1 && a->G >= 1 && a->H % a->G == 0;  // the rest is checked by g4b_attn_forward
+    const uint64_t need = (shape_ok && takes_generic_path(a)) ? 0 : g4b_attn_workspace_bytes(a->B, a->H, a->G, a->Tq, a->D, a->num_workers);
     if (need > kStaticScratchBytes)
         return fail(G4B_ERR_WORKSPACE, "this launch splits keys through %llu bytes of partials, the static scratch holds %llu; "
                     "use g4b_attn_forward with a workspace of that size",

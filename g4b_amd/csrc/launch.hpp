@@ -54,6 +54,9 @@ hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_
 // any Tq; (H/G) must divide 128; D = 512
 hipError_t launch_attn_prefill_wide(const AttnParams& p, int kv_dt, hipStream_t stream);
 
+// any Tq, any H/G, D a multiple of 8 up to 1024, kv_dt also DT_F32, STAGE_ON_BAND with its block size: plain fp32 kernel
+hipError_t launch_attn_generic(const AttnParams& p, int D, int kv_dt, int on_band_block, hipStream_t stream);
+
 // One launch for the prefill-phase slots (pp: rows > 16) and the decode-phase slots (pd: rows <= 16) of a batch.
 struct MixedPlan {
     int npx;          // prefill workgroups per XCD (grid slots; the prefill body drops the surplus)

@@ -90,6 +90,7 @@ def _bind(
     workspace=None,
     num_workers: int = 0,
     kernel_mask: int = 0,
+    on_band_block: int | None = None,
 ):
     """Validate the arguments like the reference and fill the C argument block (plus the objects it points into)."""
     assert isinstance(phase, int)  # fa2.py:653
@@ -157,6 +158,9 @@ def _bind(
     a.num_workers = int(num_workers)
     a.kernel_mask = int(kernel_mask)
     a.use_fp32_dot = 1 if use_fp32_dot else 0
+    if int(stage) == STAGE_ON_BAND and on_band_block is None:
+        raise ValueError("STAGE_ON_BAND alone needs on_band_block= (the reference's autotuned Q_BLOCKSIZE_T)")
+    a.on_band_block = 0 if on_band_block is None else int(on_band_block)
     a.scale = float(scale)
 
     if isinstance(workspace, str) and workspace != "static":
@@ -209,6 +213,7 @@ def flash_attention(
     workspace=None,
     num_workers: int = 0,
     kernel_mask: int = 0,
+    on_band_block: int | None = None,
     stream=None,
     decode_q=None,
     decode_o=None,
@@ -234,7 +239,12 @@ def flash_attention(
       with its fp32 scratchpads, ``g4b/models/gemma4e.py:606``) feeds the product with the query as
       the sum of two 16-bit operands, value and rounding error, so the scores are those of the
       unrounded query.  The products run on fp16/bf16 MFMA with fp32 accumulation either way.
-    * ``stage``: ``STAGE_CAUSAL`` or ``STAGE_FULL``.
+    * ``stage``: ``STAGE_CAUSAL``, ``STAGE_FULL``, or ``STAGE_ON_BAND`` together with ``on_band_block=``.
+
+    The tuned kernels serve head dimensions 128, 256 and 512 on fp16 / bf16 caches; other head dimensions
+    (multiples of 8 up to 1024), query-head groups that do not divide a workgroup's 128 rows, an fp32 cache
+    (the reference's ``G4B_DTKV_FP32`` switch, ``g4b/models/gemma4e.py:32``) and ``STAGE_ON_BAND`` run on a plain
+    fp32 kernel: same results, a fraction of the speed.
 
     Keyword-only extensions, with defaults that reproduce the reference:
 
@@ -246,7 +256,9 @@ def flash_attention(
       scratch array through ``g4b_attn_forward_static_scratch``: nothing is allocated, a launch whose partials exceed
       ``g4b_static_scratch_bytes()`` runs unsplit, and calls that overlap on one GPU (two streams) must not share it,
       so give every stream but one a workspace of its own; ``False`` = no scratch, never split); ``num_workers``; ``kernel_mask`` (profiling:
-      bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``.
+      bit 0 main kernel, bit 1 merge kernel, 0 = both); ``stream``; ``on_band_block`` (with ``STAGE_ON_BAND``: the
+      reference's ``Q_BLOCKSIZE_T``, ``fa2.py:56,61`` -- query ``i`` sees the keys of its own block of that many
+      positions up to itself; the reference's result for this stage depends on what its autotuner picked).
     * ``decode_q``, ``decode_o`` (``[B, H, 1, D]``), ``decode_phase``: a mixed step in one launch.  The reference
       serves a step that holds prefill-phase and decode-phase slots with two calls over the same batch tensors,
       because its kernel skips per slot on ``user_phase[b] != PHASE`` (``fa2.py:332-335``), and its scheduler avoids
@@ -262,7 +274,7 @@ def flash_attention(
     kw = dict(
         use_grouped_query_tile=use_grouped_query_tile, warp_specialize=warp_specialize, is_hopper=is_hopper,
         use_fp32_dot=use_fp32_dot, stage=stage, scale=scale, query_window=query_window, window_sizes=window_sizes,
-        num_workers=num_workers, kernel_mask=kernel_mask,
+        num_workers=num_workers, kernel_mask=kernel_mask, on_band_block=on_band_block,
     )
     if decode_q is not None or decode_o is not None:
         if partial_o is not None or partial_l is not None or partial_m is not None:

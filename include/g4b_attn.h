@@ -24,12 +24,12 @@
 extern "C" {
 #endif
 
-#define G4B_ATTN_ABI_VERSION 2
+#define G4B_ATTN_ABI_VERSION 3
 
 enum g4b_status {
     G4B_OK = 0,
     G4B_ERR_INVALID_ARGUMENT = -1, /* shape / stride / dtype / value check failed (reference: tl.static_assert) */
-    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim 64, STAGE_ON_BAND alone) */
+    G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim above 1024, a mixed launch at head_dim 128) */
     G4B_ERR_WORKSPACE = -3,        /* workspace missing or too small for the requested split-KV launch */
     G4B_ERR_LAUNCH = -4            /* the HIP runtime refused the launch (no device, bad stream, ...) */
 };
@@ -48,14 +48,20 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *   q, o          [B, H, Tq, D], any strides with last stride 1 (the engine passes permuted views
  *                 of [B, t, H, D] scratchpads, g4b/models/gemma4e.py:1031-1033); f16 / bf16 / f32.
  *   k_cache,      [B, G, KV_CTX, D], contiguous inside a slot (fa2.py:315-320), slot stride
- *   v_cache       k_stride_b / v_stride_b; f16 or bf16.
+ *   v_cache       k_stride_b / v_stride_b; f16 or bf16, or f32 (the reference's G4B_DTKV_FP32 debugging switch,
+ *                 g4b/models/gemma4e.py:32).
  *   time_dim_sizes[B] int32: tokens in the slot after this step (fa2.py:52).
  *   user_phase    [B] uint8: slots whose value differs from `phase` are skipped and their rows of
  *                 `o` are left untouched (fa2.py:332-335).
  *   ctx_window_size  W <= KV_CTX: the launch sees the last min(tds, W) keys; logical key j is ring
  *                 row (max(tds - W, 0) + j) % KV_CTX; query i is aligned with logical key
  *                 min(tds, W) - Tq + i (fa2.py:53-56,75).
- *   stage         G4B_STAGE_CAUSAL (default of the reference) or G4B_STAGE_FULL.
+ *   stage         G4B_STAGE_CAUSAL (default of the reference), G4B_STAGE_FULL, or G4B_STAGE_ON_BAND: the diagonal
+ *                 block alone (fa2.py:61,399-435), whose extent is the reference's autotuned Q_BLOCKSIZE_T and has to be
+ *                 named here.
+ *   on_band_block with G4B_STAGE_ON_BAND: Q_BLOCKSIZE_T (fa2.py:56,140-180; 1 in the reference's default configuration
+ *                 list).  Query i then sees the keys of its own block of that many positions up to itself:
+ *                 logical keys [q_t_base + (i / block) * block, q_t_base + i].  Ignored by the other stages.
  *   scale         softmax scale; the reference computes with 1.0 (fa2.py:89).
  *   query_window  0 = anchored window, the reference kernel's semantics.  > 0 additionally hides
  *                 keys with q_pos - k_pos >= query_window, the per-query sliding window of the CPU
@@ -81,6 +87,12 @@ enum g4b_phase { G4B_PHASE_UNALLOCATED = 0, G4B_PHASE_PREFILL = 1, G4B_PHASE_DEC
  *   kernel_mask   profiling aid.  0 = run every kernel of the launch.  Otherwise bit 0 selects the
  *                 main attention kernel and bit 1 the split-merge kernel, so that each can be timed
  *                 on its own; results are only complete with both.
+ *
+ * The tuned kernels serve D in {128, 256, 512} with f16 / bf16 caches, the causal and full stages and, for
+ * prefill-shaped launches ((H/G)*Tq > 16), H/G dividing 128 (64 at D = 512 with a split query): everything Gemma-4
+ * and the reference's own test list (tests/compare_scripts/test_fa2.py:51-79) use.  Any other D that is a multiple of
+ * 8 up to 1024, any other H/G, an f32 cache and G4B_STAGE_ON_BAND run on a plain fp32 kernel without matrix
+ * instructions: same results to the same tolerance, a fraction of the speed, no workspace.
  *
  * Rows whose visible key set is empty (time_dim_sizes[b] == 0 on an in-phase slot) are written
  * as zeros; the reference leaves 0/0 there and its caller ignores them (g4b/scheduler.py:142-148).
@@ -113,6 +125,7 @@ typedef struct g4b_attn_args {
     int32_t num_workers;
     int32_t kernel_mask;
     int32_t use_fp32_dot;
+    int32_t on_band_block;
     float scale;
 } g4b_attn_args;
 

@@ -45,7 +45,8 @@ def unroll_ring(cache_b: np.ndarray, tds: int, W: int) -> np.ndarray:
     return cache_b[:, rows, :]
 
 
-def visibility_mask(tds: int, W: int, Tq: int, stage: int, query_window: int | None = None) -> np.ndarray:
+def visibility_mask(tds: int, W: int, Tq: int, stage: int, query_window: int | None = None,
+                    on_band_block: int | None = None) -> np.ndarray:
     """Boolean ``[Tq, window]`` mask, vectorised form of :func:`index_spec.visible`."""
     win = ix.window_size(tds, W)
     i = np.arange(Tq)[:, None]
@@ -55,8 +56,13 @@ def visibility_mask(tds: int, W: int, Tq: int, stage: int, query_window: int | N
         m = np.ones((Tq, win), dtype=bool)
     elif stage == ix.STAGE_CAUSAL:
         m = j <= qp
+    elif stage == ix.STAGE_ON_BAND:
+        if on_band_block is None or on_band_block < 1:
+            raise ValueError("STAGE_ON_BAND alone depends on the tile size: pass on_band_block")
+        tile_start = ix.q_t_base(tds, W, Tq) + (i // on_band_block) * on_band_block  # fa2.py:56,61
+        m = (j >= tile_start) & (j <= qp)
     else:
-        raise ValueError("unsupported stage")
+        raise ValueError("unknown stage")
     if query_window is not None:
         m = m & (qp - j < query_window)
     return m
@@ -79,6 +85,7 @@ def attention_ref(
     out=None,
     dtype=np.float64,
     return_empty_rows: bool = False,
+    on_band_block: int | None = None,
 ):
     """Dense reference attention.
 
@@ -102,7 +109,7 @@ def attention_ref(
         W = int(ctx_window_size if window_sizes is None else window_sizes[b])
         k = unroll_ring(k_cache[b], tds, W)
         v = unroll_ring(v_cache[b], tds, W)
-        mask = visibility_mask(tds, W, Tq, stage, query_window)
+        mask = visibility_mask(tds, W, Tq, stage, query_window, on_band_block)
         empty[b] = ~mask.any(axis=1)
         for h in range(H):
             g = h // R  # repeat_interleave(k, H // G, 1): head h reads kv head h // R (reference_impl.py:434-435)

@@ -63,13 +63,18 @@ def q_t_base(tds: int, W: int, Tq: int) -> int:
     return window_size(tds, W) - Tq
 
 
-def visible(i: int, j: int, tds: int, W: int, Tq: int, stage: int, query_window: int | None = None) -> bool:
+def visible(i: int, j: int, tds: int, W: int, Tq: int, stage: int, query_window: int | None = None,
+            on_band_block: int | None = None) -> bool:
     """Does query ``i`` (0-based inside the launch) attend logical key ``j``?
 
     ``STAGE_FULL``: every key of the window (fa2.py:62-64, tail mask :74,:90).
     ``STAGE_CAUSAL``: keys ``j <= q_t_base + i`` (off-band range ``[0, q_tile_start)``
     plus the causally masked diagonal block, fa2.py:58-61,93-96); the union over
     tiles does not depend on the tile size.
+    ``STAGE_ON_BAND`` alone: only the diagonal block of the query's tile (fa2.py:56,61,93-96),
+    keys ``q_tile_start <= j <= q_t_base + i`` with ``q_tile_start = q_t_base +
+    (i // Q_BLOCKSIZE_T) * Q_BLOCKSIZE_T``; the tile size (``on_band_block``) is the
+    reference's autotuned constant and has to be named.
     ``query_window`` (extension; ``scripts/reference_impl.py:440-441``): additionally
     ``q_pos - k_pos < query_window``, the per-query sliding window of a one-shot
     prefill longer than the window.
@@ -81,19 +86,27 @@ def visible(i: int, j: int, tds: int, W: int, Tq: int, stage: int, query_window:
         ok = True
     elif stage == STAGE_CAUSAL:
         ok = j <= q_t_base(tds, W, Tq) + i
+    elif stage == STAGE_ON_BAND:
+        if on_band_block is None or on_band_block < 1:
+            raise ValueError("STAGE_ON_BAND alone depends on the tile size: pass on_band_block")
+        qb = q_t_base(tds, W, Tq)
+        ok = qb + (i // on_band_block) * on_band_block <= j <= qb + i
     else:
-        raise ValueError("STAGE_ON_BAND alone depends on the tile size and is not part of the contract")
+        raise ValueError("unknown stage")
     if ok and query_window is not None:
         ok = (q_t_base(tds, W, Tq) + i) - j < query_window
     return ok
 
 
-def visible_range(i: int, tds: int, W: int, Tq: int, stage: int, query_window: int | None = None) -> tuple[int, int]:
+def visible_range(i: int, tds: int, W: int, Tq: int, stage: int, query_window: int | None = None,
+                  on_band_block: int | None = None) -> tuple[int, int]:
     """Half-open logical key range ``[lo, hi)`` of query ``i`` (empty if ``hi <= lo``)."""
     win = window_size(tds, W)
     qp = q_t_base(tds, W, Tq) + i
     hi = win if stage == STAGE_FULL else min(win, qp + 1)
     lo = 0
+    if stage == STAGE_ON_BAND:
+        lo = max(0, q_t_base(tds, W, Tq) + (i // on_band_block) * on_band_block)
     if query_window is not None:
         lo = max(0, qp - query_window + 1)
     return lo, max(hi, lo)

@@ -110,15 +110,15 @@ def test_python_boundary_validates_like_the_reference(native):
         flash_attention(q, k[:, :, ::2], v[:, :, ::2], o, tds, ph, 32, PHASE_DECODE)
     with pytest.raises(ValueError):
         flash_attention(q, k, v, o, tds.long(), ph, 64, PHASE_DECODE)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError, match="on_band_block"):  # the stage alone depends on the reference's tile size
         flash_attention(q, k, v, o, tds, ph, 64, PHASE_DECODE, stage=STAGE_ON_BAND)
-    q5, k5 = torch.zeros(2, 8, 1, 192, dtype=torch.float16), torch.zeros(2, 2, 64, 192, dtype=torch.float16)
+    with pytest.raises(ValueError, match="on_band_block"):
+        flash_attention(q, k, v, o, tds, ph, 64, PHASE_DECODE, stage=STAGE_ON_BAND, on_band_block=0)
+    with pytest.raises(ValueError, match="stage"):
+        flash_attention(q, k, v, o, tds, ph, 64, PHASE_DECODE, stage=4)
+    q5, k5 = torch.zeros(2, 8, 1, 2048, dtype=torch.float16), torch.zeros(2, 2, 64, 2048, dtype=torch.float16)
     with pytest.raises(NotImplementedError, match="head_dim"):
         flash_attention(q5, k5, k5, q5.clone(), tds, ph, 64, PHASE_DECODE)
-    # prefill-shaped launches: the group size must divide the rows of a workgroup (128)
-    q6, k6 = torch.zeros(2, 6, 8, 512, dtype=torch.float16), torch.zeros(2, 2, 64, 512, dtype=torch.float16)
-    with pytest.raises(NotImplementedError, match="must divide 128"):
-        flash_attention(q6, k6, k6, q6.clone(), tds, ph, 64, PHASE_DECODE)
 
 
 def test_c_abi_rejects_bad_arguments_before_launching(native):

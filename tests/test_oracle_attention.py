@@ -158,7 +158,7 @@ def test_reference_style_slicing_equals_masked_dense(case):
     np.testing.assert_allclose(blocked, dense, rtol=2e-5, atol=2e-6)
 
 
-@pytest.mark.parametrize("stage", [ix.STAGE_CAUSAL, ix.STAGE_FULL])
+@pytest.mark.parametrize("stage", [ix.STAGE_CAUSAL, ix.STAGE_FULL, ix.STAGE_ON_BAND])
 def test_triton_tile_restatement_equals_dense(stage):
     rng = np.random.default_rng(5)
     n = 0
@@ -170,10 +170,11 @@ def test_triton_tile_restatement_equals_dense(stage):
         q, kc, vc, _ = stream_case(rng, B, H, G, Tq, D, kv_ctx, W, tds_list, dtype=np.float32)
         q *= 0.5
         phase = [1] * B
-        dense = ar.attention_ref(q, kc, vc, tds_list, phase, W, 1, stage=stage, scale=1.0)
         for BM in (1, 2, 4):
             if Tq % BM:
                 continue
+            # only the on-band stage alone depends on the tile size
+            dense = ar.attention_ref(q, kc, vc, tds_list, phase, W, 1, stage=stage, scale=1.0, on_band_block=BM)
             for BN in (1, 2, 4):
                 for S in (1, 2, 3):
                     tiles = ar.flash_tiles_ref(q, kc, vc, tds_list, phase, W, 1, stage=stage, BM=BM, BN=BN, num_splits=S)

@@ -74,9 +74,10 @@ def test_causal_visibility_equals_position_rule():
                 assert got == list(range(lo, hi))
 
 
-@pytest.mark.parametrize("stage", [ix.STAGE_CAUSAL, ix.STAGE_FULL])
+@pytest.mark.parametrize("stage", [ix.STAGE_CAUSAL, ix.STAGE_FULL, ix.STAGE_ON_BAND])
 def test_triton_program_grid_covers_exactly_the_visible_set(stage):
-    """Union over (q tile, split) programs == visible(); programs of one q tile are disjoint."""
+    """Union over (q tile, split) programs == visible(); programs of one q tile are disjoint.  STAGE_ON_BAND alone is
+    the one stage whose result depends on the tile size, which visible() therefore takes as on_band_block."""
     checked = 0
     for kv_ctx, W, tds, Tq in itertools.product([5, 8], [3, 5], [0, 1, 4, 5, 6, 9, 13], [1, 2, 4]):
         if W > kv_ctx or tds < Tq or ix.window_size(tds, W) < Tq:
@@ -93,8 +94,11 @@ def test_triton_program_grid_covers_exactly_the_visible_set(stage):
                 (i, j)
                 for i in range(Tq)
                 for j in range(ix.window_size(tds, W))
-                if ix.visible(i, j, tds, W, Tq, stage)
+                if ix.visible(i, j, tds, W, Tq, stage, on_band_block=BM)
             }
+            for i in range(Tq):
+                lo, hi = ix.visible_range(i, tds, W, Tq, stage, on_band_block=BM)
+                assert {j for (ii, j) in expect if ii == i} == set(range(lo, hi))
             assert union == expect, (kv_ctx, W, tds, Tq, BM, BN, S)
             checked += 1
     assert checked > 200

@@ -120,3 +120,43 @@ def test_generic_path_through_the_static_scratch_entry_and_plans(fa):
     torch.cuda.synchronize()
     ref = oracle(q, k, v, [80, 33], [1, 1], kv_ctx, 1, scale=0.1)
     assert_close(o.float().cpu().numpy(), ref)
+
+
+def test_fp32_cache_engine_step(fa):
+    """G4B_DTKV_FP32 end to end for one prefill chunk and one decode step: K append, V append with the fused weightless
+    RMSNorm (g4b/kernels/add_kv_to_cache.py:146-159) into fp32 rings, attention on them."""
+    from g4b_amd.kernels.add_kv_to_cache import add_kv_to_cache
+
+    B, H, G, D, t, W = 2, 8, 2, 256, 24, 40
+    T = W + t - 1
+    eps = 1e-6
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    k_cache = torch.zeros(B, G, T, D, device="cuda")
+    v_cache = torch.zeros(B, G, T, D, device="cuda")
+    ctx = [0, 0]
+    streams = [[np.zeros((G, 0, D)), np.zeros((G, 0, D))] for _ in range(B)]
+    for t_now, phase_id in ((t, 1), (t, 1), (1, 2), (1, 2)):
+        q = torch.randn(B, t_now, H, D, generator=gen).cuda().permute(0, 2, 1, 3) * 0.25
+        kx = torch.randn(B, t_now, G, D, generator=gen).cuda().permute(0, 2, 1, 3)
+        vx = torch.randn(B, t_now, G, D, generator=gen).cuda().permute(0, 2, 1, 3)
+        rs = (vx * vx).sum(-1)
+        o = torch.full((B, t_now, H, D), 777.0, device="cuda").permute(0, 2, 1, 3)
+        offs, tds, ph = i32(ctx), i32([c + t_now for c in ctx]), u8([phase_id] * B)
+        add_kv_to_cache(kx, k_cache, offs, eps, user_phase=ph, phase=phase_id)
+        add_kv_to_cache(vx, v_cache, offs, eps, rs, user_phase=ph, phase=phase_id)
+        fa.flash_attention(q, k_cache, v_cache, o, tds, ph, W, phase_id, use_fp32_dot=True, scale=1 / 8)
+        torch.cuda.synchronize()
+        vn = vx.double() * torch.rsqrt(rs.double() / D + eps)[..., None]
+        for b in range(B):
+            streams[b][0] = np.concatenate([streams[b][0], kx[b].double().cpu().numpy()], 1)
+            streams[b][1] = np.concatenate([streams[b][1], vn[b].cpu().numpy()], 1)
+            n = ctx[b] + t_now
+            lo = max(n - W, 0)
+            ks = np.repeat(streams[b][0][:, lo:n], H // G, 0)
+            vs = np.repeat(streams[b][1][:, lo:n], H // G, 0)
+            s = np.einsum("htd,hnd->htn", q[b].double().cpu().numpy(), ks) / 8
+            s = np.where(np.arange(n - t_now, n)[:, None] < np.arange(lo, n)[None, :], -np.inf, s)
+            p = np.exp(s - s.max(-1, keepdims=True))
+            ref = np.einsum("htn,hnd->htd", p / p.sum(-1, keepdims=True), vs)
+            assert_close(o[b].cpu().numpy(), ref, atol=2e-5, rtol=2e-5, what=f"slot {b} at ctx {ctx[b]}")
+        ctx = [c + t_now for c in ctx]

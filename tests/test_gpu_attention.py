@@ -464,5 +464,5 @@ def test_argument_errors_follow_the_reference(fa):
         fa.flash_attention(q, k, v, o, tds, ph, W + 1, 2)
     with pytest.raises(ValueError):  # fa2.py:293
         fa.flash_attention(q, k, v, o[:, :4], tds, ph, W, 2)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError, match="on_band_block"):  # the stage alone depends on the reference's tile size
         fa.flash_attention(q, k, v, o, tds, ph, W, 2, stage=fa.STAGE_ON_BAND)

@@ -257,3 +257,59 @@ def test_random_mixed_launch(gpu_device, n):
             assert (gp[b] == sentinel).all()
         else:
             assert (gp[b] == sentinel).all() and (gd[b] == sentinel).all(), f"mixed case {n}: idle slot {b} was written"
+
+
+N_GENERIC_CASES = 100
+
+
+@pytest.mark.parametrize("n", range(N_GENERIC_CASES))
+def test_random_launch_outside_the_tuned_shapes(gpu_device, n):
+    """The same sweep over what the tuned kernels do not cover and the plain fp32 kernel serves: head dimensions that
+    are any multiple of 8, group sizes with odd factors, fp32 caches, STAGE_ON_BAND alone with a random block size."""
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(9000 + n)
+    D = int(rng.choice([8, 16, 40, 64, 72, 96, 128, 192, 256, 320, 512, 640, 1024]))
+    R = int(rng.choice([1, 2, 3, 5, 6, 7, 12]))
+    G = int(rng.choice([1, 2, 3]))
+    H = R * G
+    Tq = int(rng.choice([1, 1, 2, 7, 16, 33, 80]))
+    kv_ctx = int(rng.integers(max(Tq, 8), 200))
+    W = int(rng.integers(max(Tq, 1), kv_ctx + 1))
+    B = int(rng.integers(1, 5))
+    phase_id = int(rng.choice([1, 2]))
+    phase = [phase_id if rng.random() < 0.75 else 0 for _ in range(B)]
+    tds = [int(rng.choice([0 if Tq == 1 else Tq, int(rng.integers(Tq, W + 1)), W, int(rng.integers(W, 4 * kv_ctx))])) for _ in range(B)]
+    stage = int(rng.choice([ix.STAGE_CAUSAL, ix.STAGE_CAUSAL, ix.STAGE_FULL, ix.STAGE_ON_BAND]))
+    block = int(rng.integers(1, Tq + 4)) if stage == ix.STAGE_ON_BAND else None
+    qwin = int(rng.integers(1, 2 * W)) if rng.random() < 0.3 else None
+    win = [int(rng.integers(Tq, W + 1)) for _ in range(B)] if rng.random() < 0.25 else None
+    cdt = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
+    qdt = torch.float32 if (cdt == torch.float32 or rng.random() < 0.4) else cdt
+    engine = rng.random() < 0.5
+    scale = float(rng.choice([1 / 16, 0.3, D**-0.5]))
+    print(dict(D=D, H=H, G=G, Tq=Tq, kv_ctx=kv_ctx, W=W, B=B, phase_id=phase_id, phase=phase, tds=tds, stage=stage, block=block,
+               qwin=qwin, win=win, cdt=cdt, qdt=qdt, engine=engine, scale=scale), flush=True)
+    gen = torch.Generator().manual_seed(9500 + n)
+    if engine:
+        q = torch.randn(B, Tq, H, D, generator=gen).to(qdt).cuda().permute(0, 2, 1, 3)
+        o = torch.full((B, Tq, H, D), 777.0, dtype=qdt, device="cuda").permute(0, 2, 1, 3)
+    else:
+        q = torch.randn(B, H, Tq, D, generator=gen).to(qdt).cuda()
+        o = torch.full((B, H, Tq, D), 777.0, dtype=qdt, device="cuda")
+    k = torch.randn(B, G, kv_ctx, D, generator=gen).to(cdt).cuda()
+    v = torch.randn(B, G, kv_ctx, D, generator=gen).to(cdt).cuda()
+    kw = dict(stage=stage, scale=scale, query_window=qwin, on_band_block=block)
+    ref = oracle(q, k, v, tds, phase, W, phase_id, window_sizes=win, **kw)
+    if win is not None:
+        kw["window_sizes"] = i32(win)
+    fa2.flash_attention(q, k, v, o, i32(tds), u8(phase), W, phase_id, use_fp32_dot=True, **kw)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if cdt == torch.bfloat16 else {}
+    sentinel = torch.tensor(777.0, dtype=qdt).float().item()
+    for b in range(B):
+        if phase[b] == phase_id:
+            assert_close(got[b], ref[b], what=f"case {n} slot {b}", **tol)
+        else:
+            assert (got[b] == sentinel).all(), f"case {n}: off-phase slot {b} was written"

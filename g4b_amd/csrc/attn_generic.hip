@@ -18,26 +18,6 @@ namespace {
 constexpr int GEN_MAX_D = 1024;
 constexpr int GEN_WAVES = 4;
 
-G4B_DEV void load8_f32(const void* base, int64_t elem_off, int dt, float (&x)[8]) {
-    if (dt == DT_F32) {
-        const f4* p = reinterpret_cast<const f4*>(static_cast<const float*>(base) + elem_off);
-        const f4 a = p[0], b = p[1];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            x[i] = a[i];
-            x[4 + i] = b[i];
-        }
-    } else {
-        const u4 raw = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = raw[i];
-            x[2 * i] = (dt == DT_F16) ? F16::lo(w) : BF16::lo(w);
-            x[2 * i + 1] = (dt == DT_F16) ? F16::hi(w) : BF16::hi(w);
-        }
-    }
-}
-
 G4B_DEV float wave_max64(float v) {
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) v = fmaxf(v, __shfl_xor(v, s));
@@ -88,7 +68,7 @@ __global__ __launch_bounds__(64 * GEN_WAVES) void attn_generic_kernel(const Attn
     const int nchunk = D >> 3;  // 8-column pieces of a row
     if (tid < nchunk) {
         float x[8];
-        load8_f32(p.q, (int64_t)b * p.q_s[0] + (int64_t)h * p.q_s[1] + (int64_t)i * p.q_s[2] + tid * 8, p.q_dt, x);
+        load_f32<8>(p.q, (int64_t)b * p.q_s[0] + (int64_t)h * p.q_s[1] + (int64_t)i * p.q_s[2] + tid * 8, p.q_dt, x);
 #pragma unroll
         for (int e = 0; e < 8; ++e) sm.q[tid * 8 + e] = x[e] * p.c;
     }
@@ -124,7 +104,7 @@ __global__ __launch_bounds__(64 * GEN_WAVES) void attn_generic_kernel(const Attn
         float s0 = 0.f, s1 = 0.f;
         for (int c = 0; c < nchunk; ++c) {
             float kx[8];
-            load8_f32(krow, c * 8, kv_dt, kx);
+            load_f32<8>(krow, c * 8, kv_dt, kx);
             const f4 qa = *reinterpret_cast<const f4*>(&sm.q[c * 8]);
             const f4 qc = *reinterpret_cast<const f4*>(&sm.q[c * 8 + 4]);
 #pragma unroll
@@ -156,7 +136,7 @@ __global__ __launch_bounds__(64 * GEN_WAVES) void attn_generic_kernel(const Attn
                     const int c = c0 + u * 64;
                     if (u < cpl && c < nchunk) {
                         float vx[8];
-                        load8_f32(vrow, c * 8, kv_dt, vx);
+                        load_f32<8>(vrow, c * 8, kv_dt, vx);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) acc[u][e] = fmaf(pk, vx[e], acc[u][e]);
                     }

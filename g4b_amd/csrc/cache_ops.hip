@@ -7,14 +7,16 @@
 
 namespace g4b {
 
-// One thread moves 8 consecutive elements; a workgroup of 256 threads covers 2048 elements of the
-// [G, t, D] block of one slot, so writes to a cache row are 16-byte vectors and fully coalesced.
+// One thread moves N consecutive elements, 16 bytes of the wider of the two types (N = 4 when the scratchpad or the
+// cache is fp32, else 8), so a wave reads and writes contiguous runs; a workgroup of 256 threads covers 256 * N
+// elements of the [G, t, D] block of one slot.
+template <int N>
 __global__ __launch_bounds__(256) void kv_append_kernel(const KvAppendParams p) {
     const int b = blockIdx.y;
     if (p.phase_arr && p.phase_arr[(int64_t)b * p.ph_s] != (uint8_t)p.phase) return;
     const int64_t off = p.off_is_i64 ? static_cast<const int64_t*>(p.offsets)[(int64_t)b * p.off_s]
                                      : (int64_t) static_cast<const int32_t*>(p.offsets)[(int64_t)b * p.off_s];
-    const int segs = p.D / 8;
+    const int segs = p.D / N;
     const int64_t n = (int64_t)p.G * p.t * segs;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= n) return;
@@ -24,35 +26,25 @@ __global__ __launch_bounds__(256) void kv_append_kernel(const KvAppendParams p) 
     int64_t row = (tt + off) % p.T;
     if (row < 0) row += p.T;
 
-    const int64_t xo = (int64_t)b * p.x_s[0] + (int64_t)g * p.x_s[1] + (int64_t)tt * p.x_s[2] + seg * 8;
-    float v[8];
-    if (p.x_dt == DT_F32) {
-        const f4* src = reinterpret_cast<const f4*>(static_cast<const float*>(p.x) + xo);
-        f4 a = src[0], c = src[1];
-        v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3];
-        v[4] = c[0]; v[5] = c[1]; v[6] = c[2]; v[7] = c[3];
-    } else {
-        u4 raw = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(p.x) + xo);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[2 * i] = p.x_dt == DT_F16 ? F16::lo(raw[i]) : BF16::lo(raw[i]);
-            v[2 * i + 1] = p.x_dt == DT_F16 ? F16::hi(raw[i]) : BF16::hi(raw[i]);
-        }
-    }
+    const int64_t xo = (int64_t)b * p.x_s[0] + (int64_t)g * p.x_s[1] + (int64_t)tt * p.x_s[2] + seg * N;
+    float v[N];
+    load_f32<N>(p.x, xo, p.x_dt, v);
     if (p.x_rsos) {
         const float r = p.x_rsos[(int64_t)b * p.rsos_s[0] + (int64_t)g * p.rsos_s[1] + (int64_t)tt * p.rsos_s[2]];
         const float inv = 1.0f / __builtin_sqrtf(r / (float)p.D + p.eps);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] *= inv;
+        for (int i = 0; i < N; ++i) v[i] *= inv;
     }
-    const int64_t co = (int64_t)b * p.cache_sb + ((int64_t)g * p.T + row) * p.D + seg * 8;
-    store8(p.cache, co, p.cache_dt, v);
+    const int64_t co = (int64_t)b * p.cache_sb + ((int64_t)g * p.T + row) * p.D + seg * N;
+    store_n<N>(p.cache, co, p.cache_dt, v);
 }
 
 hipError_t launch_kv_append(const KvAppendParams& p, hipStream_t stream) {
-    const int64_t n = (int64_t)p.G * p.t * (p.D / 8);
+    const int N = (p.x_dt == DT_F32 || p.cache_dt == DT_F32) ? 4 : 8;
+    const int64_t n = (int64_t)p.G * p.t * (p.D / N);
     dim3 grid((unsigned)((n + 255) / 256), p.B);
-    hipLaunchKernelGGL(kv_append_kernel, grid, dim3(256), 0, stream, p);
+    if (N == 4) hipLaunchKernelGGL(kv_append_kernel<4>, grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(kv_append_kernel<8>, grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

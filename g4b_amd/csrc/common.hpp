@@ -155,6 +155,47 @@ G4B_DEV void store4(void* base, int64_t elem_off, int dt, f4 v) {
     }
 }
 
+// N consecutive elements (4 or 8; dtype chosen at run time) as floats: one 16-byte load per four fp32 values or eight
+// 16-bit ones, so that the lanes of a wave read one contiguous run.
+template <int N>
+G4B_DEV void load_f32(const void* base, int64_t elem_off, int dt, float (&v)[N]) {
+    static_assert(N == 4 || N == 8, "4 or 8 elements");
+    if (dt == DT_F32) {
+        const f4* src = reinterpret_cast<const f4*>(static_cast<const float*>(base) + elem_off);
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            const f4 a = src[q];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[4 * q + i] = a[i];
+        }
+    } else {
+        uint32_t raw[N / 2];
+        if constexpr (N == 8) {
+            const u4 r = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) raw[i] = r[i];
+        } else {
+            const u2 r = *reinterpret_cast<const u2*>(static_cast<const uint16_t*>(base) + elem_off);
+            raw[0] = r[0];
+            raw[1] = r[1];
+        }
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            v[2 * i] = dt == DT_F16 ? F16::lo(raw[i]) : BF16::lo(raw[i]);
+            v[2 * i + 1] = dt == DT_F16 ? F16::hi(raw[i]) : BF16::hi(raw[i]);
+        }
+    }
+}
+template <int N>
+G4B_DEV void store_n(void* base, int64_t elem_off, int dt, const float (&v)[N]) {
+    if constexpr (N == 8) {
+        store8(base, elem_off, dt, v);
+    } else {
+        const f4 x = {v[0], v[1], v[2], v[3]};
+        store4(base, elem_off, dt, x);
+    }
+}
+
 // ---- wave64 cross-lane -----------------------------------------------------------------------
 template <int CTRL>
 G4B_DEV float dpp_f(float x) {

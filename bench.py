@@ -577,6 +577,61 @@ def measure(wl: Workload, steps: int, warmup: int):
     return res
 
 
+def sample_power(wl, seconds):
+    """Board power and shader clock while ``wl`` runs back to back for ``seconds``: power from the amdgpu hwmon node
+    (microwatts, sampled between batches of launches), the shader clock from ``rocm-smi --showclocks`` (a child
+    process per sample).  The second half of the samples is averaged, after the power controller has settled."""
+    import glob
+    import re
+    import subprocess
+    import threading
+
+    import torch
+
+    def read(path):
+        try:
+            with open(path) as f:
+                return float(f.read().strip())
+        except (OSError, ValueError):
+            return None
+
+    nodes = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")
+    power_file = next((f"{n}/{leaf}" for n in nodes for leaf in ("power1_input", "power1_average") if read(f"{n}/{leaf}") is not None), None)
+    cap = next((read(f"{n}/power1_cap") for n in nodes if read(f"{n}/power1_cap") is not None), None)
+    watts, mhz, stop = [], [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            if power_file:
+                w = read(power_file)
+                if w is not None:
+                    watts.append(w / 1e6)
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+                m = re.search(r"sclk clock level: \S+ \((\d+)Mhz\)", out)
+                if m:
+                    mhz.append(int(m.group(1)))
+            except (OSError, subprocess.SubprocessError):
+                stop.wait(0.05)
+
+    th = threading.Thread(target=sampler)
+    th.start()
+    t0, n = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            wl.launch()
+        n += 20
+        torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    stop.set()
+    th.join()
+    half = lambda xs: xs[len(xs) // 2:]  # noqa: E731
+    mean = lambda xs: round(sum(xs) / len(xs), 1) if xs else None  # noqa: E731
+    return {"seconds": round(elapsed, 2), "ms_per_launch": round(elapsed / n * 1e3, 4), "watts": mean(half(watts)),
+            "cap_watts": None if cap is None else round(cap / 1e6, 1), "sclk_mhz": mean(half(mhz)),
+            "power_samples": len(watts), "clock_samples": len(mhz)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -592,6 +647,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic, used to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--sample-power", type=float, default=0.0, metavar="SECONDS",
+                    help="afterwards run the primary workload back to back for SECONDS and report board power and "
+                         "shader clock under it (\"power\" in the JSON line)")
     args = ap.parse_args()
     if args.traffic_from:
         print(json.dumps(traffic_from_counters(args.traffic_from), indent=1, sort_keys=True))
@@ -641,6 +699,10 @@ def main():
         return c
 
     cpu = None if args.no_cpu_baseline else cpu_baseline_of(wl)
+    power = None
+    if args.sample_power > 0:
+        power = sample_power(wl, args.sample_power)
+        log(f"power under {wl.name}: {power}")
 
     extra = {}
     if not args.no_extra:
@@ -690,6 +752,8 @@ def main():
         "device": props.name,
         "extra": extra,
     }
+    if power is not None:
+        line["power"] = power
     print(json.dumps(line), flush=True)
 
 

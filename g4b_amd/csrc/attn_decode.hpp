@@ -18,6 +18,9 @@
 // score layout of the first MFMA is the B-operand layout of the second, with the key order of the
 // contraction chosen to match.  V^T operands are built with an in-lane 8x8 16-bit transpose.
 #pragma once
+#ifndef G4B_DEC_LD
+#define G4B_DEC_LD ld16_stream
+#endif
 #include "common.hpp"
 
 namespace g4b {
@@ -127,7 +130,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
         for (int tau = 0; tau < NT; ++tau) {
             const uint32_t ro = key_off(jb + tau * KT + m16 / CL);
 #pragma unroll
-            for (int c = 0; c < NC; ++c) kreg[tau][c] = ld16(kbase, ro + (uint32_t)(cls + CL * g4 + 4 * CL * c) * 16u);
+            for (int c = 0; c < NC; ++c) kreg[tau][c] = G4B_DEC_LD(kbase, ro + (uint32_t)(cls + CL * g4 + 4 * CL * c) * 16u);
         }
     };
     auto load_v = [&](int t) {
@@ -136,7 +139,7 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
         for (int s = 0; s < 8; ++s) {
             const uint32_t ro = key_off(jb + (s / E) * KT + g4 * E + (s % E));
 #pragma unroll
-            for (int dc = 0; dc < DC; ++dc) vreg[dc][s] = ld16(vbase, ro + (uint32_t)(m16 + 16 * dc) * 16u);
+            for (int dc = 0; dc < DC; ++dc) vreg[dc][s] = G4B_DEC_LD(vbase, ro + (uint32_t)(m16 + 16 * dc) * 16u);
         }
     };
 

@@ -69,6 +69,10 @@ struct BF16 {
 G4B_DEV u4 ld16(const void* base, uint32_t byte_off) {
     return *reinterpret_cast<const u4*>(static_cast<const char*>(base) + byte_off);
 }
+// The same load marked non-temporal: the line is read once (a KV stream) and need not stay in the caches.
+G4B_DEV u4 ld16_stream(const void* base, uint32_t byte_off) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u4*>(static_cast<const char*>(base) + byte_off));
+}
 G4B_DEV u4 ld16(const void* base, int64_t byte_off) {
     return *reinterpret_cast<const u4*>(static_cast<const char*>(base) + byte_off);
 }

@@ -295,10 +295,11 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
 // half gets what lets its stream run at full rate, the chunk the rest.
 namespace {
 constexpr int kMixedCus = 256;
-// Decode workgroups asked for by default: four one-wave workers each at head dimension 256 (the stream reaches its
-// rate with 320..384 workers); one four-wave worker each at 512, whose waves keep half as many bytes in flight and
-// need more of the chip (measured on the benchmark's global layers: 96 workgroups 381 us, 128 327 us, 160 380 us).
-constexpr int kMixedDecodeBlocks = 80;
+// Decode workgroups asked for by default (the prefill half then takes as many whole key splits as fit and the decode
+// half what is left): four one-wave workers each at head dimension 256, one four-wave worker each at 512.  Measured
+// on the benchmark's global layers, main kernel: head dim 256 with 96 decode workgroups (five key splits of the chunk)
+// 151 us, 100..128 (four splits) 138..147 us, 160 169 us; head dim 512 with 104 348 us, 120 320 us, 128 312 us, 136 348 us.
+constexpr int kMixedDecodeBlocks = 112;
 constexpr int kMixedDecodeBlocksWide = 112;
 
 struct MixedShape {

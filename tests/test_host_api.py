@@ -239,10 +239,10 @@ def test_mixed_launch_is_validated_before_launching(native):
                         decode_o=torch.zeros(B, H, 1, 128, dtype=torch.float16))
     # sizing: the chunk's partials ((slot, split) pairs x H x t x (D + 2) floats, rounded up to 256 bytes) followed by the
     # decode partials ((workers + B*G) x rows x (D + 2) floats).  64-token chunks bring 2 tiles x 2 kv heads = 4 workgroups
-    # per slot; the default share-out leaves 256 - 80 = 176 units to the chunk -> 44 pairs, and the decode half gets the
-    # remaining 80 workgroups of four workers.
+    # per slot; the default share-out leaves 256 - 112 = 144 units to the chunk -> 36 pairs, and the decode half gets the
+    # remaining 112 workgroups of four workers.
     n = mixed_workspace_bytes(B, H, G, t, 1, D, T, T)
-    assert n == 44 * H * t * (D + 2) * 4 + (320 + B * G) * 4 * (D + 2) * 4
+    assert n == 36 * H * t * (D + 2) * 4 + (448 + B * G) * 4 * (D + 2) * 4
     # a short window takes the one-workgroup-per-pair decode path: no decode partials, 256 - B*G units for the chunk
     n_swa = mixed_workspace_bytes(B, H, G, t, 1, D, 512 + t - 1, 512)
     assert n_swa == 63 * H * t * (D + 2) * 4

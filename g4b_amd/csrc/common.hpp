@@ -131,55 +131,70 @@ G4B_DEV void load8_split(const void* base, int64_t elem_off, int dt, u4& hi, u4&
     }
 }
 
+// A vector load / store that is marked non-temporal when NT: data touched once (scratchpads read by one pass, a KV
+// stream) then passes through the caches without displacing what others re-read.
+template <bool NT, class V>
+G4B_DEV V ld_vec(const V* p) {
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+template <bool NT, class V>
+G4B_DEV void st_vec(V* p, V v) {
+    if constexpr (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
 // Store eight consecutive output elements (dtype chosen at run time) from eight floats.
+template <bool NT = false>
 G4B_DEV void store8(void* base, int64_t elem_off, int dt, const float (&v)[8]) {
     if (dt == DT_F32) {
         f4* p = reinterpret_cast<f4*>(static_cast<float*>(base) + elem_off);
         f4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
-        p[0] = a;
-        p[1] = b;
+        st_vec<NT>(p, a);
+        st_vec<NT>(p + 1, b);
     } else if (dt == DT_F16) {
         u4 r = {F16::pack2(v[0], v[1]), F16::pack2(v[2], v[3]), F16::pack2(v[4], v[5]), F16::pack2(v[6], v[7])};
-        *reinterpret_cast<u4*>(static_cast<uint16_t*>(base) + elem_off) = r;
+        st_vec<NT>(reinterpret_cast<u4*>(static_cast<uint16_t*>(base) + elem_off), r);
     } else {
         u4 r = {BF16::pack2(v[0], v[1]), BF16::pack2(v[2], v[3]), BF16::pack2(v[4], v[5]), BF16::pack2(v[6], v[7])};
-        *reinterpret_cast<u4*>(static_cast<uint16_t*>(base) + elem_off) = r;
+        st_vec<NT>(reinterpret_cast<u4*>(static_cast<uint16_t*>(base) + elem_off), r);
     }
 }
 
+template <bool NT = false>
 G4B_DEV void store4(void* base, int64_t elem_off, int dt, f4 v) {
     if (dt == DT_F32) {
-        *reinterpret_cast<f4*>(static_cast<float*>(base) + elem_off) = v;
+        st_vec<NT>(reinterpret_cast<f4*>(static_cast<float*>(base) + elem_off), v);
     } else if (dt == DT_F16) {
         u2 r = {F16::pack2(v[0], v[1]), F16::pack2(v[2], v[3])};
-        *reinterpret_cast<u2*>(static_cast<uint16_t*>(base) + elem_off) = r;
+        st_vec<NT>(reinterpret_cast<u2*>(static_cast<uint16_t*>(base) + elem_off), r);
     } else {
         u2 r = {BF16::pack2(v[0], v[1]), BF16::pack2(v[2], v[3])};
-        *reinterpret_cast<u2*>(static_cast<uint16_t*>(base) + elem_off) = r;
+        st_vec<NT>(reinterpret_cast<u2*>(static_cast<uint16_t*>(base) + elem_off), r);
     }
 }
 
 // N consecutive elements (4 or 8; dtype chosen at run time) as floats: one 16-byte load per four fp32 values or eight
 // 16-bit ones, so that the lanes of a wave read one contiguous run.
-template <int N>
+template <int N, bool NT = false>
 G4B_DEV void load_f32(const void* base, int64_t elem_off, int dt, float (&v)[N]) {
     static_assert(N == 4 || N == 8, "4 or 8 elements");
     if (dt == DT_F32) {
         const f4* src = reinterpret_cast<const f4*>(static_cast<const float*>(base) + elem_off);
 #pragma unroll
         for (int q = 0; q < N / 4; ++q) {
-            const f4 a = src[q];
+            const f4 a = ld_vec<NT>(src + q);
 #pragma unroll
             for (int i = 0; i < 4; ++i) v[4 * q + i] = a[i];
         }
     } else {
         uint32_t raw[N / 2];
         if constexpr (N == 8) {
-            const u4 r = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off);
+            const u4 r = ld_vec<NT>(reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off));
 #pragma unroll
             for (int i = 0; i < 4; ++i) raw[i] = r[i];
         } else {
-            const u2 r = *reinterpret_cast<const u2*>(static_cast<const uint16_t*>(base) + elem_off);
+            const u2 r = ld_vec<NT>(reinterpret_cast<const u2*>(static_cast<const uint16_t*>(base) + elem_off));
             raw[0] = r[0];
             raw[1] = r[1];
         }
@@ -190,13 +205,13 @@ G4B_DEV void load_f32(const void* base, int64_t elem_off, int dt, float (&v)[N])
         }
     }
 }
-template <int N>
+template <int N, bool NT = false>
 G4B_DEV void store_n(void* base, int64_t elem_off, int dt, const float (&v)[N]) {
     if constexpr (N == 8) {
-        store8(base, elem_off, dt, v);
+        store8<NT>(base, elem_off, dt, v);
     } else {
         const f4 x = {v[0], v[1], v[2], v[3]};
-        store4(base, elem_off, dt, x);
+        store4<NT>(base, elem_off, dt, x);
     }
 }
 

@@ -138,9 +138,45 @@ def check_wait_discipline() -> dict:
     return seen
 
 
+def check_stream_loads() -> dict:
+    """The decode kernels read K and V with non-temporal loads (a fifth of their throughput hangs on it) and q with
+    ordinary ones.  The marking is metadata the optimiser may drop when it merges loads, so the generated assembly is
+    checked: every worker / pair instantiation must carry `global_load_dwordx4 ... nt` for its stream.
+
+    Returns {kernel symbol: (non-temporal 16-byte loads, ordinary 16-byte loads)}."""
+    import re
+    import tempfile
+
+    seen = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        out = Path(tmp) / "attn_decode.s"
+        cmd = [hipcc(), *COMMON_FLAGS, *DEVICE_FLAGS, "-S", "--cuda-device-only", str(CSRC / "attn_decode.hip"), "-o", str(out)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc -S failed on attn_decode.hip:\n{res.stderr}")
+        cur = None
+        for line in out.read_text().splitlines():
+            m = re.match(r"(_ZN3g4b\d+attn_decode_(?:worker|pair)\w*):", line)
+            if m:
+                cur = m.group(1)
+                seen[cur] = [0, 0]
+            elif line.startswith(".Lfunc_end"):
+                cur = None
+            elif cur and "global_load_dwordx4" in line:
+                seen[cur][0 if re.search(r"\bnt\b", line) else 1] += 1
+    if not seen:
+        raise RuntimeError("no decode kernel found in the assembly of attn_decode.hip")
+    for sym, (nt, plain) in seen.items():
+        if nt < 24 or nt <= plain:
+            raise RuntimeError(f"{sym}: {nt} non-temporal and {plain} ordinary 16-byte loads; the K/V stream lost its nt marking")
+    return {k: tuple(v) for k, v in seen.items()}
+
+
 if __name__ == "__main__":
     path = build(verbose="--verbose" in sys.argv)
     print(path)
     if "--check-waits" in sys.argv:
         for sym, n in check_wait_discipline().items():
             print(f"wait discipline ok: {sym} ({n} MFMAs)")
+        for sym, (nt, plain) in check_stream_loads().items():
+            print(f"stream loads ok: {sym} ({nt} non-temporal, {plain} ordinary)")

@@ -211,6 +211,16 @@ def test_pipelined_kernels_keep_foreign_memory_traffic_out_of_their_wait_regions
     assert all(n >= 48 for n in seen.values()), seen
 
 
+def test_decode_stream_keeps_its_non_temporal_loads():
+    """K and V of a decode launch are read once, with `global_load_dwordx4 ... nt`; the marking is optimiser metadata
+    (merging such a load with an ordinary one drops it without a word), so the generated assembly is scanned."""
+    from g4b_amd.build import check_stream_loads
+
+    seen = check_stream_loads()
+    # worker: head dims 128 / 256 / 512 x three row classes x fp16 / bf16 x query rounded or split; pair: 128 / 256
+    assert len(seen) == 36 + 24, sorted(seen)
+
+
 def test_mixed_launch_is_validated_before_launching(native):
     """g4b_attn_forward_mixed checks both argument blocks and their agreement on the host (no GPU needed)."""
     from g4b_amd.kernels.fa2 import PHASE_DECODE, PHASE_PREFILL, flash_attention, mixed_workspace_bytes

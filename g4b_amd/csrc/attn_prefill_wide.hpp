@@ -319,7 +319,9 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
                     *reinterpret_cast<f4*>(p.part_o + prow * D + half * 256 + pc * 4) = v;
                 } else {
                     const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
-                    store4(p.o, off + half * 256 + pc * 4, p.o_dt, v);
+                    // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2
+                    // (S = 8192 0.5 % faster, the 512-key sliding window 3.7 %; the same hint on the Q loads cost 1.3 .. 4 %)
+                    store4<true>(p.o, off + half * 256 + pc * 4, p.o_dt, v);
                 }
             }
         }

@@ -77,17 +77,30 @@ G4B_DEV u4 ld16(const void* base, int64_t byte_off) {
     return *reinterpret_cast<const u4*>(static_cast<const char*>(base) + byte_off);
 }
 
+// A vector load / store that is marked non-temporal when NT: data touched once (scratchpads read by one pass, a KV
+// stream) then passes through the caches without displacing what others re-read.
+template <bool NT, class V>
+G4B_DEV V ld_vec(const V* p) {
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+template <bool NT, class V>
+G4B_DEV void st_vec(V* p, V v) {
+    if constexpr (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
 // Eight consecutive elements of a q/x row (dtype chosen at run time) as eight MFMA operand
 // elements of type T, optionally pre-multiplied.
-template <class T>
+template <class T, bool NT = false>
 G4B_DEV u4 load8_as(const void* base, int64_t elem_off, int dt) {
     if (dt == DT_F32) {
         const f4* p = reinterpret_cast<const f4*>(static_cast<const float*>(base) + elem_off);
-        f4 a = p[0], b = p[1];
+        f4 a = ld_vec<NT>(p), b = ld_vec<NT>(p + 1);
         u4 r = {T::pack2(a[0], a[1]), T::pack2(a[2], a[3]), T::pack2(b[0], b[1]), T::pack2(b[2], b[3])};
         return r;
     }
-    u4 raw = *reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off);
+    u4 raw = ld_vec<NT>(reinterpret_cast<const u4*>(static_cast<const uint16_t*>(base) + elem_off));
     if (dt == T::dt) return raw;
     u4 r;
     if (dt == DT_F16) {
@@ -129,19 +142,6 @@ G4B_DEV void load8_split(const void* base, int64_t elem_off, int dt, u4& hi, u4&
         hi[i] = h;
         lo[i] = T::pack2(x[2 * i] - T::lo(h), x[2 * i + 1] - T::hi(h));
     }
-}
-
-// A vector load / store that is marked non-temporal when NT: data touched once (scratchpads read by one pass, a KV
-// stream) then passes through the caches without displacing what others re-read.
-template <bool NT, class V>
-G4B_DEV V ld_vec(const V* p) {
-    if constexpr (NT) return __builtin_nontemporal_load(p);
-    else return *p;
-}
-template <bool NT, class V>
-G4B_DEV void st_vec(V* p, V v) {
-    if constexpr (NT) __builtin_nontemporal_store(v, p);
-    else *p = v;
 }
 
 // Store eight consecutive output elements (dtype chosen at run time) from eight floats.

@@ -271,21 +271,27 @@ def flash_attention(
     Returns ``(None, None)`` in place of the reference's two launch handles, which its callers
     ignore (``g4b/models/gemma4e.py:593-607``).
     """
-    kw = dict(
+    a, _keep, entry = _bind_call(
+        q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, partial_o, partial_l, partial_m,
         use_grouped_query_tile=use_grouped_query_tile, warp_specialize=warp_specialize, is_hopper=is_hopper,
         use_fp32_dot=use_fp32_dot, stage=stage, scale=scale, query_window=query_window, window_sizes=window_sizes,
-        num_workers=num_workers, kernel_mask=kernel_mask, on_band_block=on_band_block,
+        workspace=workspace, num_workers=num_workers, kernel_mask=kernel_mask, on_band_block=on_band_block,
+        decode_q=decode_q, decode_o=decode_o, decode_phase=decode_phase,
     )
+    _native.check(entry(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    return None, None
+
+
+def _bind_call(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase, partial_o=None, partial_l=None,
+               partial_m=None, *, workspace=None, decode_q=None, decode_o=None, decode_phase=PHASE_DECODE, **kw):
+    """Arguments of :func:`flash_attention` (without ``stream``) -> (argument block, objects to keep alive, entry point)."""
     if decode_q is not None or decode_o is not None:
         if partial_o is not None or partial_l is not None or partial_m is not None:
             raise ValueError("a mixed launch takes its scratch through workspace=, not partial_o/l/m")
-        a, _keep, entry = _bind_mixed(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase,
-                                      decode_q, decode_o, decode_phase, workspace, **kw)
-    else:
-        a, _keep, entry = _bind(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase,
-                                partial_o, partial_l, partial_m, workspace=workspace, **kw)
-    _native.check(entry(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
-    return None, None
+        return _bind_mixed(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase,
+                           decode_q, decode_o, decode_phase, workspace, **kw)
+    return _bind(q, k_cache, v_cache, o, time_dim_sizes, user_phase, ctx_window_size, phase,
+                 partial_o, partial_l, partial_m, workspace=workspace, **kw)
 
 
 class AttentionPlan:
@@ -308,14 +314,7 @@ class AttentionPlan:
 
 
 def plan_flash_attention(*args, **kwargs) -> AttentionPlan:
-    """Same arguments as :func:`flash_attention` (without ``stream``); returns an :class:`AttentionPlan`."""
+    """Same arguments as :func:`flash_attention`, positional or by keyword (``stream`` is ignored: it is given to
+    ``launch``); returns an :class:`AttentionPlan`."""
     kwargs.pop("stream", None)
-    if kwargs.get("decode_q") is not None or kwargs.get("decode_o") is not None:
-        decode_q, decode_o = kwargs.pop("decode_q", None), kwargs.pop("decode_o", None)
-        decode_phase = kwargs.pop("decode_phase", PHASE_DECODE)
-        workspace = kwargs.pop("workspace", None)
-        a, keep, entry = _bind_mixed(*args[:8], decode_q, decode_o, decode_phase, workspace, **kwargs)
-    else:
-        kwargs.pop("decode_q", None), kwargs.pop("decode_o", None), kwargs.pop("decode_phase", None)
-        a, keep, entry = _bind(*args, **kwargs)
-    return AttentionPlan(a, keep, entry)
+    return AttentionPlan(*_bind_call(*args, **kwargs))

@@ -183,3 +183,22 @@ def test_mixed_step_recorded_into_a_graph(fa):
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(eager.tds, replayed.tds) and torch.equal(eager.od, replayed.od) and torch.equal(eager.op, replayed.op)
+
+
+def test_plan_takes_the_arguments_by_keyword(fa):
+    """plan_flash_attention binds like flash_attention: every argument may come by keyword, also for a mixed launch."""
+    B, t, kv_ctx = 3, 64, 700
+    qp, qd, k, v = make_batch(B, t, kv_ctx, seed=36)
+    tds, phase = [600, 300 + t, 50], [2, 1, 2]
+    ws = torch.empty(fa.mixed_workspace_bytes(B, H, G, t, 1, D, kv_ctx, kv_ctx), dtype=torch.uint8, device="cuda")
+    op, od = torch.full_like(qp, 777.0), torch.full_like(qd, 777.0)
+    plan = fa.plan_flash_attention(q=qp, k_cache=k, v_cache=v, o=op, time_dim_sizes=i32(tds), user_phase=u8(phase),
+                                   ctx_window_size=kv_ctx, phase=ix.PHASE_PREFILL, scale=1 / 16, workspace=ws, decode_q=qd,
+                                   decode_o=od, stream=None)
+    plan.launch()
+    torch.cuda.synchronize()
+    ref_p = oracle(qp, k, v, tds, phase, kv_ctx, 1, scale=1 / 16)
+    ref_d = oracle(qd, k, v, tds, phase, kv_ctx, 2, scale=1 / 16)
+    assert_close(op[1].float().cpu().numpy(), ref_p[1])
+    for b in (0, 2):
+        assert_close(od[b].float().cpu().numpy(), ref_d[b])

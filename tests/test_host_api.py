@@ -93,6 +93,22 @@ def _decode_args():
     return q, k, k.clone(), q.clone(), torch.zeros(2, dtype=torch.int32), torch.zeros(2, dtype=torch.uint8)
 
 
+def test_integration_stub_lists_the_argument_block_as_the_library_has_it(native):
+    """The ctypes structure printed in INTEGRATION.md is what a maintainer would paste: same fields, order and types as
+    the structure this package binds (which the test above holds against the header)."""
+    import re
+    from pathlib import Path
+
+    text = (Path(__file__).resolve().parent.parent / "INTEGRATION.md").read_text()
+    body = text[text.index("class g4b_attn_args(C.Structure)"):text.index("lib.g4b_attn_forward.argtypes")]
+    doc = []
+    for name, ctype, length in re.findall(r'\("(\w+)", C\.(c_\w+)(?: \* (\d+))?\)', body):
+        doc.append((name, getattr(ctypes, ctype), int(length or 0)))  # c_int32 and c_int are one type
+    ours = [(name, getattr(ctype, "_type_", ctype) if hasattr(ctype, "_length_") else ctype, getattr(ctype, "_length_", 0))
+            for name, ctype in native.AttnArgs._fields_]
+    assert doc == ours
+
+
 def test_python_boundary_validates_like_the_reference(native):
     from g4b_amd.kernels.fa2 import PHASE_DECODE, STAGE_CAUSAL, STAGE_FULL, STAGE_ON_BAND, flash_attention
 

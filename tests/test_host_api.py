@@ -94,8 +94,8 @@ def _decode_args():
 
 
 def test_integration_stub_lists_the_argument_block_as_the_library_has_it(native):
-    """The ctypes structure printed in the integration notes at the repository root is what a maintainer would paste: same fields, order and types as
-    the structure this package binds (which the test above holds against the header)."""
+    """The ctypes structure printed in the integration notes at the repository root is what a maintainer would paste:
+    same fields, order and types as the structure this package binds (which the test above holds against the header)."""
     import re
     from pathlib import Path
 

@@ -30,18 +30,24 @@ CASES = {
     "chunk_on_context": (2, 8, 2, 40, 128, 103, 64, [40, 167], [1, 1], 1, ix.STAGE_CAUSAL, 1 / 16, None),
     "full_stage": (2, 4, 4, 24, 128, 24, 24, [24, 41], [1, 1], 1, ix.STAGE_FULL, 1.0, None),
     "per_query_window": (1, 8, 2, 72, 128, 72, 72, [72], [1], 1, ix.STAGE_CAUSAL, 1 / 16, 17),
+    # the diagonal block alone, for a tile size (Q_BLOCKSIZE_T, fa2.py:56,61) of 16 query positions
+    "on_band_block16": (2, 8, 2, 48, 128, 120, 96, [48, 200], [1, 1], 1, ix.STAGE_ON_BAND, 1 / 16, None, 16),
 }
 
 
 def build(name):
-    B, H, G, Tq, D, kv_ctx, W, tds, phase_arr, phase, stage, scale, qw = CASES[name]
+    B, H, G, Tq, D, kv_ctx, W, tds, phase_arr, phase, stage, scale, qw, *rest = CASES[name]
+    band = rest[0] if rest else None
     rng = np.random.default_rng(sum(map(ord, name)))
     q = rng.standard_normal((B, H, Tq, D)).astype(np.float16)
     k = rng.standard_normal((B, G, kv_ctx, D)).astype(np.float16)
     v = rng.standard_normal((B, G, kv_ctx, D)).astype(np.float16)
     out0 = np.full((B, H, Tq, D), 777.0)
-    o = ar.attention_ref(q, k, v, tds, phase_arr, W, phase, stage=stage, scale=scale, query_window=qw, out=out0.copy())
+    o = ar.attention_ref(q, k, v, tds, phase_arr, W, phase, stage=stage, scale=scale, query_window=qw, out=out0.copy(),
+                         on_band_block=band)
+    extra = {} if band is None else {"on_band_block": np.int32(band)}
     return dict(
+        **extra,
         q=q, k_cache=k, v_cache=v, time_dim_sizes=np.array(tds, np.int32), user_phase=np.array(phase_arr, np.uint8),
         ctx_window_size=np.int32(W), phase=np.int32(phase), stage=np.int32(stage), scale=np.float32(scale),
         query_window=np.int32(0 if qw is None else qw), expected=o.astype(np.float32),

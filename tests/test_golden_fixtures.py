@@ -22,10 +22,11 @@ def test_fixtures_present():
 def test_oracle_reproduces_fixture(path):
     f = np.load(path)
     qw = int(f["query_window"]) or None
+    band = int(f["on_band_block"]) if "on_band_block" in f else None
     out = np.full(f["expected"].shape, 777.0)
     got = ar.attention_ref(
         f["q"], f["k_cache"], f["v_cache"], f["time_dim_sizes"], f["user_phase"], int(f["ctx_window_size"]),
-        int(f["phase"]), stage=int(f["stage"]), scale=float(f["scale"]), query_window=qw, out=out,
+        int(f["phase"]), stage=int(f["stage"]), scale=float(f["scale"]), query_window=qw, out=out, on_band_block=band,
     )
     assert np.array_equal(got.astype(np.float32), f["expected"])
     # skipped slots keep the sentinel, everything else is finite
@@ -61,7 +62,8 @@ def test_kernels_match_fixture(gpu_device, path, split):
     extra = {} if split or decode_shaped else {"workspace": False}
     flash_attention(
         q, k, v, o, t("time_dim_sizes"), t("user_phase"), int(f["ctx_window_size"]), int(f["phase"]), *parts,
-        stage=int(f["stage"]), scale=float(f["scale"]), query_window=int(f["query_window"]) or None, **extra,
+        stage=int(f["stage"]), scale=float(f["scale"]), query_window=int(f["query_window"]) or None,
+        on_band_block=int(f["on_band_block"]) if "on_band_block" in f else None, **extra,
     )
     torch.cuda.synchronize()
     assert_close(o.float().cpu().numpy(), f["expected"], what=os.path.basename(path))

@@ -244,6 +244,25 @@ class SingleDecode(Workload):
     def launch(self, i=0, kernel_mask=0):
         self.plans[(i % self.copies, kernel_mask)].launch()
 
+    def graph_replay_ms(self, replays=20):
+        """The same launches recorded once into a graph (all cache copies, in order) and replayed, which is how the
+        engine runs its decode step (g4b/lifecycle.py:29-53): wall time per launch without the host's share."""
+        import torch
+
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for c in range(self.copies):
+                self.plans[(c, 0)].launch()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / (replays * self.copies)
+
     def cpu_sample(self):
         from oracle import attention_ref as ar
 
@@ -728,6 +747,8 @@ def main():
                      "TFLOP/s": round(r["TFLOPs"], 2), "roofline": r["roofline"]}
             if isinstance(w, MixedStep):
                 entry["detail"] = w.detail
+            if hasattr(w, "graph_replay_ms"):
+                entry["graph_replay_ms_per_step"] = round(w.graph_replay_ms(), 4)
             if name == "prefill_causal_8192" and not args.no_cpu_baseline:
                 # the prefill half of the metric carries its own CPU baseline (a three-second sample)
                 entry["cpu_baseline"] = cpu_baseline_of(w, 3.0)

@@ -79,7 +79,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     const PfMap map = pf_map(n_active * p.G * nsplit, pf_ranks(nsplit, nq_tiles));
     if (bid >= map.grid) return;
     int head, rank;
-    pf_item(map, bid, head, rank);
+    pf_item(map, bid, head, rank, p.qwin > 0);
     if (rank >= map.nq) return;
     // Unsplit launches give a workgroup two query tiles of its head, the rank-th from the end and the rank-th from the
     // start: under the causal mask their key ranges add up to the same length for every workgroup, and the second

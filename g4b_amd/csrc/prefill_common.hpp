@@ -25,7 +25,7 @@ G4B_DEV PfWork pf_select_work(const AttnParams& p, int bid, int rows_per_workgro
     const PfMap map = pf_map(n_active * p.G * w.nsplit, paired ? pf_ranks(w.nsplit, w.nq_tiles) : w.nq_tiles);
     if (bid >= map.grid) return w;
     int head;
-    pf_item(map, bid, head, w.rank);
+    pf_item(map, bid, head, w.rank, p.qwin > 0);
     if (w.rank >= map.nq) return w;
     w.split = head % w.nsplit;
     w.g = (head / w.nsplit) % p.G;

@@ -29,11 +29,15 @@ __host__ __device__ inline PfMap pf_map(int heads, int nq) {
     }
     return m;
 }
-__host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int& rank) {
+// blocked: a per-query window shorter than the span makes a query tile read only the keys around it, so the XCDs
+// that share a head take contiguous runs of its query tiles (each then fetches its own part of K/V) instead of taking
+// the tiles in turn (which suits the causal prefix that every tile reads).
+__host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int& rank, bool blocked = false) {
     const int x = f & 7, j = f >> 3;
-    if (map.mode == 1) {  // heads divide 8: 8 / heads XCDs share a head and take its query tiles in turn
+    if (map.mode == 1) {  // heads divide 8: 8 / heads XCDs share a head
+        const int share = 8 / map.heads;
         head = x % map.heads;
-        rank = j * (8 / map.heads) + x / map.heads;
+        rank = blocked ? (x / map.heads) * (map.grid >> 3) + j : j * share + x / map.heads;
     } else if (map.mode == 2) {  // 8 divides heads: every XCD owns heads / 8 heads
         head = (j % (map.heads / 8)) * 8 + x;
         rank = j / (map.heads / 8);

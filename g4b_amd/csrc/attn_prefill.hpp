@@ -85,8 +85,11 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     // start: under the causal mask their key ranges add up to the same length for every workgroup, and the second
     // item starts without a new workgroup having to be placed, scan the slots and set its staging up.
     const int ipw = pf_items_per_workgroup(nsplit, nq_tiles);
-    const int qtile_first = nq_tiles - 1 - rank;
-    const int n_items = (ipw == 2 && rank != qtile_first) ? 2 : 1;
+    // (with a per-query window every tile has the same work: neighbours are paired instead, whose key ranges overlap)
+    const bool near_pair = ipw == 2 && p.qwin > 0;
+    const int qtile_first = near_pair ? min(2 * rank + 1, nq_tiles - 1) : nq_tiles - 1 - rank;
+    const int qtile_second = near_pair ? 2 * rank : rank;
+    const int n_items = (ipw == 2 && qtile_second != qtile_first) ? 2 : 1;
     const int split = head % nsplit, g = (head / nsplit) % p.G, a_idx = head / (nsplit * p.G);
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);  // workgroup-uniform
 
@@ -216,7 +219,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     for (int item = 0; item < 2; ++item) {
     if (item >= n_items) break;
     if (item > 0) __syncthreads();  // every wave has read its rows of the previous item back from LDS
-    const int qtile = item == 0 ? qtile_first : rank;
+    const int qtile = item == 0 ? qtile_first : qtile_second;
     const int tok0 = qtile * TOKB;
     const int tok_last = min(tok0 + TOKB, Tq) - 1;
     // key range of the workgroup and the range that every row shares

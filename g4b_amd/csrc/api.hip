@@ -94,11 +94,23 @@ uint64_t decode_slots(int B, int G, int nw) { return (uint64_t)nw + (uint64_t)B 
 constexpr int kPrefillFillWorkgroups = 256;
 constexpr int kPrefillMaxSplitSlots = 64;
 int prefill_rows_per_workgroup(int /*D*/) { return 128; }
+// A slot that brings at least half as many query tiles as the chip has compute units is not split tile by tile; the
+// 128 / 256 kernel then still has only a quarter to a half of the units busy with its pairs of query tiles, and cuts
+// the key tiles of every pair into two or three equal spans instead (measured, one slot, causal from an empty cache:
+// S = 3072 95 -> 64 us, S = 4096 119 -> 89 us; for shorter prompts, which the tile-by-tile split already serves, it
+// measured worse: S = 1024 25 -> 32 us).  The 512 kernel gives every workgroup one query tile.
+bool prefill_pair_split(int H, int G, int Tq, int D) {
+    const int R = H / G, bm = prefill_rows_per_workgroup(D);
+    if (D == 512 || R < 1 || bm % R) return false;
+    const int tokb = bm / R, nq = (Tq + tokb - 1) / tokb;
+    return (int64_t)nq * G * 2 > kPrefillFillWorkgroups && (int64_t)((nq + 1) / 2) * G * 2 <= kPrefillFillWorkgroups;
+}
 int prefill_split_slots(int H, int G, int Tq, int D) {
     const int R = H / G, bm = prefill_rows_per_workgroup(D);
     if (R < 1 || bm % R) return 0;
     const int tokb = bm / R;
-    const int64_t per_slot = (int64_t)((Tq + tokb - 1) / tokb) * G;  // workgroups one slot brings
+    const int nq = (Tq + tokb - 1) / tokb;
+    const int64_t per_slot = (int64_t)(prefill_pair_split(H, G, Tq, D) ? (nq + 1) / 2 : nq) * G;  // workgroups one slot brings
     const int64_t slots = kPrefillFillWorkgroups / per_slot;
     if (slots < 2) return 0;
     return (int)(slots < kPrefillMaxSplitSlots ? slots : kPrefillMaxSplitSlots);
@@ -278,6 +290,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
                             (unsigned long long)a->workspace_bytes, (unsigned long long)need);
             if (!aligned16(a->workspace)) return fail(G4B_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
             p.split_slots = prefill_split_slots(a->H, a->G, a->Tq, a->D);
+            p.pair_split = prefill_pair_split(a->H, a->G, a->Tq, a->D) ? 1 : 0;
             p.part_o = static_cast<float*>(a->workspace);
             p.part_ml = p.part_o + (uint64_t)p.split_slots * a->H * a->Tq * a->D;
         }

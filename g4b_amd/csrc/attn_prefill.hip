@@ -4,20 +4,25 @@
 
 namespace g4b {
 
-template <int D, class T, bool QS>
-static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
+template <int D, class T, bool QS, bool PS>
+static hipError_t launch_prefill_ps(const AttnParams& p, hipStream_t stream) {
     const int TOKB = PF_BM / p.R;
     const int slots = p.part_o ? p.split_slots : 1;
     const int blocks = prefill_grid(p);
     dim3 grid(blocks);
     const int smem = 4 * PfSmem<D>::TILE;
     static uint64_t attr_done = 0;
-    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T, QS>), smem, attr_done);
+    hipError_t e = allow_dynamic_smem(reinterpret_cast<const void*>(&attn_prefill_kernel<D, T, QS, PS>), smem, attr_done);
     if (e != hipSuccess) return e;
-    if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_kernel<D, T, QS>), grid, dim3(256), smem, stream, p);
+    if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_kernel<D, T, QS, PS>), grid, dim3(256), smem, stream, p);
     if (slots > 1 && (p.kernel_mask & 2))
         hipLaunchKernelGGL((attn_prefill_combine<D>), dim3(prefill_combine_grid(p)), dim3(256), 0, stream, p);
     return hipGetLastError();
+}
+
+template <int D, class T, bool QS>
+static hipError_t launch_prefill_t(const AttnParams& p, hipStream_t stream) {
+    return p.pair_split ? launch_prefill_ps<D, T, QS, true>(p, stream) : launch_prefill_ps<D, T, QS, false>(p, stream);
 }
 
 hipError_t launch_attn_prefill(const AttnParams& p, int D, int kv_dt, hipStream_t stream) {

@@ -51,7 +51,10 @@ struct PfSmem {
 // B operands, the rounded value and its rounding error, against the same K fragments.
 // The body of workgroup `bid` of a launch (256 threads).  smem: 4 * PfSmem<D>::TILE bytes of LDS, 16-byte aligned;
 // sh_scan: 8 ints of LDS.
-template <int D, class T, bool QS>
+// PS: the launch pairs query tiles although it splits keys (AttnParams::pair_split); a variant of its own because the
+// few scalars it adds to the set-up of a query tile change the register allocation of the main loop (the unsplit
+// S = 8192 launch measured 0.5 % slower with them compiled in).
+template <int D, class T, bool QS, bool PS = false>
 G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* sh_scan) {
     using SM = PfSmem<D>;
     constexpr int KSTEPS = D / 16;               // contraction steps of the first product
@@ -76,7 +79,8 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     if (n_active == 0) return;
     const int nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
     const int nq_tiles = (Tq + TOKB - 1) / TOKB;
-    const PfMap map = pf_map(n_active * p.G * nsplit, pf_ranks(nsplit, nq_tiles));
+    constexpr bool pair_split = PS;
+    const PfMap map = pf_map(n_active * p.G * nsplit, pf_ranks(nsplit, nq_tiles, pair_split));
     if (bid >= map.grid) return;
     int head, rank;
     pf_item(map, bid, head, rank, p.qwin > 0);
@@ -84,7 +88,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     // Unsplit launches give a workgroup two query tiles of its head, the rank-th from the end and the rank-th from the
     // start: under the causal mask their key ranges add up to the same length for every workgroup, and the second
     // item starts without a new workgroup having to be placed, scan the slots and set its staging up.
-    const int ipw = pf_items_per_workgroup(nsplit, nq_tiles);
+    const int ipw = pf_items_per_workgroup(nsplit, nq_tiles, pair_split);
     // (with a per-query window every tile has the same work: neighbours are paired instead, whose key ranges overlap)
     const bool near_pair = ipw == 2 && p.qwin > 0;
     const int qtile_first = near_pair ? min(2 * rank + 1, nq_tiles - 1) : nq_tiles - 1 - rank;
@@ -94,6 +98,25 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);  // workgroup-uniform
 
     const SlotInfo si = slot_info(p, b);
+
+    // Key splits: the key tiles of the workgroup's query tiles -- the first tile's, then the second's -- are one list
+    // that is cut into nsplit equal spans; this workgroup owns span `split` (tiles [span0, span1) of the list).
+    auto tile_span = [&](int qtile, int& count) {
+        const int t0 = qtile * TOKB, t1 = min(t0 + TOKB, Tq) - 1;
+        int lo, hi, unused;
+        row_range(p, si, t0, lo, unused);
+        row_range(p, si, t1, unused, hi);
+        count = hi > lo ? (hi - 1) / PF_BN - lo / PF_BN + 1 : 0;
+    };
+    int n_first = 0, n_second = 0, span0 = 0, span1 = 0;
+    if constexpr (PS) {
+        if (nsplit > 1) {
+            tile_span(qtile_first, n_first);
+            if (n_items == 2) tile_span(qtile_second, n_second);
+        }
+        span0 = split * (n_first + n_second) / nsplit;
+        span1 = (split + 1) * (n_first + n_second) / nsplit;
+    }
 
     const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;
     const char* vbase = static_cast<const char*>(p.v) + ((int64_t)b * p.v_sb + (int64_t)g * KV_CTX * D) * 2;
@@ -243,16 +266,26 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;  // exponent reference in log2 units (scaled), running sum (this lane's keys)
+    bool have_keys = !PS;                  // the span holds tiles of this query tile
+    bool whole = false;                    // ... all of them: the rows are final and go straight to o
 
     if (hi_wg > lo_wg) {
         // this workgroup's share of the item's key tiles
         int kt0 = lo_wg / PF_BN, kt1 = (hi_wg - 1) / PF_BN;
         if (nsplit > 1) {
-            const int n = kt1 - kt0 + 1;
-            kt1 = kt0 + (split + 1) * n / nsplit - 1;
-            kt0 = kt0 + split * n / nsplit;
+            if constexpr (PS) {
+                const int base = item == 0 ? 0 : n_first, n = item == 0 ? n_first : n_second;
+                whole = span0 <= base && span1 - base >= n;  // the span holds every key tile of this query tile
+                kt1 = kt0 + min(span1 - base, n) - 1;
+                kt0 = kt0 + max(span0 - base, 0);
+            } else {
+                const int n = kt1 - kt0 + 1;
+                kt1 = kt0 + (split + 1) * n / nsplit - 1;
+                kt0 = kt0 + split * n / nsplit;
+            }
         }
         if (kt1 >= kt0) {
+        if constexpr (PS) have_keys = true;
 
         // ---- prologue: K(kt0), K(kt0+1), V(kt0) staged; S(kt0) computed --------------------------------
         stage_whole_tile(kt0, false, 0);
@@ -459,7 +492,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     // pieces XOR-swizzled with the row so that neither side conflicts) and stores whole rows: one instruction covers
     // 64 / (D/4) complete rows instead of touching 32 rows at 8 or 16 bytes each.
     const float l_tot = half_swap_sum(l_run);
-    const bool partial = nsplit > 1;
+    const bool partial = nsplit > 1 && !whole;
     const float inv = partial ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);
     char* wbase = smem + wave * (32 * D * 4);
 #pragma unroll
@@ -470,11 +503,11 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
             const int pc = 8 * dt + 2 * q4 + h2;
             *reinterpret_cast<f4*>(wbase + n32 * (D * 4) + ((pc ^ (n32 & 15)) * 16)) = v;
         }
-    if (partial && h2 == 0 && row_ok) {
-        // (reference, sum) of this key split's rows
+    if (nsplit > 1 && h2 == 0 && row_ok) {
+        // (reference, sum) of this key split's rows; a negative sum tells the merge kernel that the row is final
         const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hh)) * Tq + ti;
         p.part_ml[prow * 2] = (m_run == -INFINITY) ? 0.f : m_run;
-        p.part_ml[prow * 2 + 1] = l_tot;
+        p.part_ml[prow * 2 + 1] = whole ? -1.f : l_tot;
     }
     constexpr int LPR = D / 4;       // lanes that cover a row, 16 bytes of fp32 each
     constexpr int RPI = 64 / LPR;    // rows per store instruction
@@ -485,7 +518,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
         const int rr = wave * 32 + row;
         const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
         const f4 v = *reinterpret_cast<const f4*>(wbase + row * (D * 4) + ((pc ^ (row & 15)) * 16));
-        if (tr < Tq) {
+        if (tr < Tq && (have_keys || !partial)) {  // a span without tiles of this query tile leaves (0, 0) in part_ml only
             if (partial) {
                 // un-normalised partial result of this key split: [pair][H][Tq][D] fp32
                 const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
@@ -501,11 +534,11 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     }
 }
 
-template <int D, class T, bool QS>
+template <int D, class T, bool QS, bool PS = false>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const AttnParams p) {
     extern __shared__ __align__(16) char smem[];
     __shared__ int sh_scan[8];
-    prefill_body<D, T, QS>(p, blockIdx.x, smem, sh_scan);
+    prefill_body<D, T, QS, PS>(p, blockIdx.x, smem, sh_scan);
 }
 
 }  // namespace g4b

@@ -327,6 +327,7 @@ struct AttnParams {
     int32_t split_slots;  // prefill: (active slot, key split) pairs the partial buffers hold; <= 1 = never split
     int32_t kernel_mask;  // bit 0: main kernel, bit 1: merge kernel
     int32_t q_split;      // 1: a query wider than the cache type enters K Q^T as a hi + lo pair of operands
+    int32_t pair_split;   // 1: a prefill launch that splits keys still pairs query tiles (prefill_map.hpp)
     float c;     // softmax scale * log2(e)
 };
 

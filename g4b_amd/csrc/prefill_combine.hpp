@@ -18,12 +18,21 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
         if (t >= p.Tq) continue;
         float ms[NS], ls[NS];
         f4 ov[NS];
+        bool final_row = false;  // a workgroup that held every key tile of the row's query tile has written o itself
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             const int64_t prow = ((int64_t)(a_idx * nsplit + min(s, nsplit - 1)) * p.H + h) * p.Tq + t;  // clamped, masked below
             ms[s] = p.part_ml[prow * 2];
             ls[s] = (s < nsplit) ? p.part_ml[prow * 2 + 1] : 0.f;
-            ov[s] = *reinterpret_cast<const f4*>(p.part_o + prow * D + d0);
+            final_row |= ls[s] < 0.f;
+        }
+        if (final_row) continue;
+        // spans without key tiles of the row's query tile left (0, 0) and no sums: only what was written is read
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int64_t prow = ((int64_t)(a_idx * nsplit + min(s, nsplit - 1)) * p.H + h) * p.Tq + t;
+            const f4 zero = {0.f, 0.f, 0.f, 0.f};
+            ov[s] = ls[s] > 0.f ? *reinterpret_cast<const f4*>(p.part_o + prow * D + d0) : zero;
         }
         float mref = -INFINITY;
 #pragma unroll

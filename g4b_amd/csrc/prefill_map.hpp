@@ -47,13 +47,18 @@ __host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int&
     }
 }
 
-// Query tiles per workgroup of the 128/256 kernel.  A launch that does not split keys pairs the r-th heaviest query
-// tile of a head with the r-th lightest in one workgroup: equal work for every workgroup under the causal mask, and
-// half as many workgroup starts.
-__host__ __device__ inline int pf_items_per_workgroup(int nsplit, int nq) { return (nsplit == 1 && nq >= 2) ? 2 : 1; }
+// Query tiles per workgroup of the 128/256 kernel.  A launch pairs the r-th heaviest query tile of a head with the
+// r-th lightest in one workgroup: equal work for every pair under the causal mask, and half as many workgroup starts.
+// When the pairs are fewer than the compute units, the key tiles of a pair -- the heavy tile's, then the light
+// tile's -- are one list that is cut into nsplit equal spans, one workgroup each (pair_split; without it a launch
+// that splits keys gives every workgroup one query tile and a uniform share of its keys, which suits query tiles of
+// equal work: a chunk on a long context).
+__host__ __device__ inline int pf_items_per_workgroup(int nsplit, int nq, bool pair_split = false) {
+    return ((nsplit == 1 || pair_split) && nq >= 2) ? 2 : 1;
+}
 // Ranks (workgroups) per head: query tiles, or pairs of them.
-__host__ __device__ inline int pf_ranks(int nsplit, int nq) {
-    return pf_items_per_workgroup(nsplit, nq) == 2 ? (nq + 1) / 2 : nq;
+__host__ __device__ inline int pf_ranks(int nsplit, int nq, bool pair_split = false) {
+    return pf_items_per_workgroup(nsplit, nq, pair_split) == 2 ? (nq + 1) / 2 : nq;
 }
 
 // Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on
@@ -68,10 +73,10 @@ inline int prefill_grid(const AttnParams& p, int bm = PF_BM, bool paired = true)
     const int n_small = slots / 2 + 1 > 8 ? slots / 2 + 1 : 8;
     for (int n = 1; n <= n_small && n <= p.B; ++n) {
         const int ns = prefill_splits(slots, n);
-        const int g = pf_map(n * p.G * ns, paired ? pf_ranks(ns, nq) : nq).grid;
+        const int g = pf_map(n * p.G * ns, paired ? pf_ranks(ns, nq, p.pair_split != 0) : nq).grid;
         blocks = g > blocks ? g : blocks;
     }
-    const int g_all = pf_map(p.B * p.G * prefill_splits(slots, p.B), paired ? pf_ranks(prefill_splits(slots, p.B), nq) : nq).grid;
+    const int g_all = pf_map(p.B * p.G * prefill_splits(slots, p.B), paired ? pf_ranks(prefill_splits(slots, p.B), nq, p.pair_split != 0) : nq).grid;
     return g_all > blocks ? g_all : blocks;
 }
 

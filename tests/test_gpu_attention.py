@@ -466,3 +466,40 @@ def test_argument_errors_follow_the_reference(fa):
         fa.flash_attention(q, k, v, o[:, :4], tds, ph, W, 2)
     with pytest.raises(ValueError, match="on_band_block"):  # the stage alone depends on the reference's tile size
         fa.flash_attention(q, k, v, o, tds, ph, W, 2, stage=fa.STAGE_ON_BAND)
+
+
+@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("case", ["from_scratch", "on_context", "two_active", "per_query_window", "full_stage", "bf16"])
+def test_prefill_pairs_of_query_tiles_cut_into_key_spans(fa, D, case):
+    """A slot that brings between a quarter and a half of the chip's compute units in pairs of query tiles: the key tiles
+    of every pair (heavy tile, then light tile) are cut into two or three equal spans, one workgroup each; a tile that
+    lies wholly in one span is written straight to o, the others are merged.  H/G = 16 makes a query tile 8 tokens, so
+    1000 tokens are 125 tiles = 63 pairs per kv head."""
+    print(f"pair split {case} D={D}", flush=True)
+    H, G, Tq, kv_ctx = 32, 2, 1000, 1300
+    B = 3 if case == "two_active" else 2
+    dtype = torch.bfloat16 if case == "bf16" else torch.float16
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=len(case) + D, dtype=dtype)
+    tds = {"from_scratch": [Tq, 5], "on_context": [kv_ctx + 300, 5], "two_active": [Tq, 1250, Tq + 7]}.get(case, [Tq + 130, 5])
+    phase = [1, 1, 0] if case == "two_active" else [1, 2]
+    kw = {}
+    if case == "per_query_window":
+        kw["query_window"] = 200
+    if case == "full_stage":
+        kw["stage"] = ix.STAGE_FULL
+    assert fa.workspace_bytes(B, H, G, Tq, D) > 0
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), kv_ctx, 1, scale=D**-0.5, **kw)
+    torch.cuda.synchronize()
+    ref = oracle(q, k, v, tds, phase, kv_ctx, 1, scale=D**-0.5, **kw)
+    got = o.float().cpu().numpy()
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if case == "bf16" else {}
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(got[b], ref[b], what=f"slot {b}", **tol)
+        else:
+            assert (got[b] == 777.0).all()
+    # the same launch without key splits
+    o2 = torch.full_like(o, 777.0)
+    fa.flash_attention(q, k, v, o2, i32(tds), u8(phase), kv_ctx, 1, scale=D**-0.5, workspace=False, **kw)
+    torch.cuda.synchronize()
+    assert (o.float() - o2.float()).abs().max().item() <= (6e-2 if case == "bf16" else 4e-3)

@@ -476,6 +476,7 @@ WORKLOADS = {
     "decode_batched_d512": lambda dev: BatchedDecode(dev, B=32, swa_every=0, dim=512, name="decode_batched_b32_d512"),
     "decode_single": lambda dev: SingleDecode(dev),
     "prefill_causal_2048": lambda dev: Prefill(dev, 2048),
+    "prefill_causal_4096": lambda dev: Prefill(dev, 4096),  # between the configs: pairs of query tiles cut into key spans
     "prefill_causal_8192": lambda dev: Prefill(dev, 8192),
     "prefill_swa_8192": lambda dev: Prefill(dev, 8192, query_window=512),
     "prefill_causal_8192_d512": lambda dev: Prefill(dev, 8192, dim=512),

@@ -80,7 +80,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     const int nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
     const int nq_tiles = (Tq + TOKB - 1) / TOKB;
     constexpr bool pair_split = PS;
-    const PfMap map = pf_map(n_active * p.G * nsplit, pf_ranks(nsplit, nq_tiles, pair_split));
+    const PfMap map = pf_map(n_active * p.G * nsplit, pf_ranks(nsplit, nq_tiles, pair_split, n_active * p.G));
     if (bid >= map.grid) return;
     int head, rank;
     pf_item(map, bid, head, rank, p.qwin > 0);
@@ -88,7 +88,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     // Unsplit launches give a workgroup two query tiles of its head, the rank-th from the end and the rank-th from the
     // start: under the causal mask their key ranges add up to the same length for every workgroup, and the second
     // item starts without a new workgroup having to be placed, scan the slots and set its staging up.
-    const int ipw = pf_items_per_workgroup(nsplit, nq_tiles, pair_split);
+    const int ipw = pf_items_per_workgroup(nsplit, nq_tiles, pair_split, n_active * p.G);
     // (with a per-query window every tile has the same work: neighbours are paired instead, whose key ranges overlap)
     const bool near_pair = ipw == 2 && p.qwin > 0;
     const int qtile_first = near_pair ? min(2 * rank + 1, nq_tiles - 1) : nq_tiles - 1 - rank;

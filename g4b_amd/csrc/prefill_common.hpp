@@ -22,7 +22,7 @@ G4B_DEV PfWork pf_select_work(const AttnParams& p, int bid, int rows_per_workgro
     const int tokb = rows_per_workgroup / p.R;
     w.nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
     w.nq_tiles = (p.Tq + tokb - 1) / tokb;
-    const PfMap map = pf_map(n_active * p.G * w.nsplit, paired ? pf_ranks(w.nsplit, w.nq_tiles) : w.nq_tiles);
+    const PfMap map = pf_map(n_active * p.G * w.nsplit, paired ? pf_ranks(w.nsplit, w.nq_tiles, false, n_active * p.G) : w.nq_tiles);
     if (bid >= map.grid) return w;
     int head;
     pf_item(map, bid, head, w.rank, p.qwin > 0);

@@ -53,12 +53,18 @@ __host__ __device__ inline void pf_item(const PfMap& map, int f, int& head, int&
 // tile's -- are one list that is cut into nsplit equal spans, one workgroup each (pair_split; without it a launch
 // that splits keys gives every workgroup one query tile and a uniform share of its keys, which suits query tiles of
 // equal work: a chunk on a long context).
-__host__ __device__ inline int pf_items_per_workgroup(int nsplit, int nq, bool pair_split = false) {
-    return ((nsplit == 1 || pair_split) && nq >= 2) ? 2 : 1;
+// A launch whose query tiles are no more than the compute units (PF_FILL) stays one tile per workgroup: pairs would
+// leave half of the chip idle (eight slots with a 512-token chunk each are 256 tiles).  unsplit_heads = in-phase slots
+// x kv heads.
+constexpr int PF_FILL = 256;
+__host__ __device__ inline int pf_items_per_workgroup(int nsplit, int nq, bool pair_split, int unsplit_heads) {
+    if (nq < 2) return 1;
+    if (pair_split) return 2;
+    return (nsplit == 1 && unsplit_heads * nq > PF_FILL) ? 2 : 1;
 }
 // Ranks (workgroups) per head: query tiles, or pairs of them.
-__host__ __device__ inline int pf_ranks(int nsplit, int nq, bool pair_split = false) {
-    return pf_items_per_workgroup(nsplit, nq, pair_split) == 2 ? (nq + 1) / 2 : nq;
+__host__ __device__ inline int pf_ranks(int nsplit, int nq, bool pair_split, int unsplit_heads) {
+    return pf_items_per_workgroup(nsplit, nq, pair_split, unsplit_heads) == 2 ? (nq + 1) / 2 : nq;
 }
 
 // Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on
@@ -68,15 +74,18 @@ inline int prefill_grid(const AttnParams& p, int bm = PF_BM, bool paired = true)
     const int nq = (p.Tq + tokb - 1) / tokb;
     const int slots = p.part_o ? p.split_slots : 1;
     int blocks = 0;
-    // keys are only split while 2 * n <= slots and the XCD-sharing map (up to 8 heads) rounds its grid up; beyond both
-    // the grid grows with n, so n = B is the largest
-    const int n_small = slots / 2 + 1 > 8 ? slots / 2 + 1 : 8;
-    for (int n = 1; n <= n_small && n <= p.B; ++n) {
+    auto grid_for = [&](int n) {
         const int ns = prefill_splits(slots, n);
-        const int g = pf_map(n * p.G * ns, paired ? pf_ranks(ns, nq, p.pair_split != 0) : nq).grid;
-        blocks = g > blocks ? g : blocks;
-    }
-    const int g_all = pf_map(p.B * p.G * prefill_splits(slots, p.B), paired ? pf_ranks(prefill_splits(slots, p.B), nq, p.pair_split != 0) : nq).grid;
+        return pf_map(n * p.G * ns, paired ? pf_ranks(ns, nq, p.pair_split != 0, n * p.G) : nq).grid;
+    };
+    // keys are only split while 2 * n <= slots and the XCD-sharing map (up to 8 heads) rounds its grid up; beyond both
+    // the grid grows with n except where the tiles start to be paired (n * G * nq passing PF_FILL), so the candidates
+    // are the small n, the last n before the pairing, and n = B
+    const int n_small = slots / 2 + 1 > 8 ? slots / 2 + 1 : 8;
+    for (int n = 1; n <= n_small && n <= p.B; ++n) blocks = grid_for(n) > blocks ? grid_for(n) : blocks;
+    const int n_unpaired = PF_FILL / (p.G * nq);
+    if (n_unpaired >= 1) blocks = grid_for(n_unpaired < p.B ? n_unpaired : p.B) > blocks ? grid_for(n_unpaired < p.B ? n_unpaired : p.B) : blocks;
+    const int g_all = grid_for(p.B);
     return g_all > blocks ? g_all : blocks;
 }
 

@@ -515,3 +515,25 @@ def test_prefill_3000_token_prompt_at_the_benchmark_head_shape(fa):
     torch.cuda.synchronize()
     ref = oracle(q, k, v, [Tq], [1], Tq, 1, scale=1 / 16)
     assert_close(o.float().cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("n_active", [5, 8, 9])
+def test_batch_of_prefill_chunks_one_query_tile_per_workgroup(fa, n_active):
+    """Several slots with a 512-token chunk each (what the scheduler's prefill step looks like): too many for key splits,
+    and up to eight of them are no more query tiles (8 x 2 kv heads x 16) than the chip has compute units, so every
+    workgroup takes one tile; nine are paired again."""
+    print(f"batch of chunks, {n_active} in phase", flush=True)
+    B, H, G, Tq, D, kv_ctx = 10, 8, 2, 512, 256, 900
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=n_active)
+    phase = [1 if b < n_active else 2 for b in range(B)]
+    tds = [Tq + 37 * b for b in range(B)]
+    ws = torch.empty(fa.workspace_bytes(B, H, G, Tq, D), dtype=torch.uint8, device="cuda")
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), kv_ctx, 1, scale=1 / 16, workspace=ws)
+    torch.cuda.synchronize()
+    ref = oracle(q, k, v, tds, phase, kv_ctx, 1, scale=1 / 16)
+    got = o.float().cpu().numpy()
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(got[b], ref[b], what=f"slot {b}")
+        else:
+            assert (got[b] == 777.0).all()

@@ -313,3 +313,49 @@ def test_random_launch_outside_the_tuned_shapes(gpu_device, n):
             assert_close(got[b], ref[b], what=f"case {n} slot {b}", **tol)
         else:
             assert (got[b] == sentinel).all(), f"case {n}: off-phase slot {b} was written"
+
+
+N_WORK_CASES = 16
+
+
+@pytest.mark.parametrize("n", range(N_WORK_CASES))
+def test_random_prefill_work_distribution(gpu_device, n):
+    """Prefill launches large enough to reach every way the query tiles are dealt to workgroups: one tile each, pairs,
+    pairs cut into key spans, uniform key splits, with any number of slots in phase -- against the fp64 oracle."""
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(12000 + n)
+    D = int(rng.choice([128, 256]))
+    R = int(rng.choice([4, 8, 16]))
+    G = int(rng.choice([1, 2, 4])) if R < 16 else int(rng.choice([1, 2]))
+    H = R * G
+    Tq = int(rng.integers(200, 1101))
+    kv_ctx = int(rng.integers(Tq, Tq + 500))
+    W = int(rng.integers(Tq, kv_ctx + 1))
+    B = int(rng.integers(1, 7))
+    phase = [1 if rng.random() < 0.7 else 2 for _ in range(B)]
+    phase[int(rng.integers(0, B))] = 1
+    tds = [int(rng.choice([Tq, int(rng.integers(Tq, W + 1)), int(rng.integers(W, 3 * kv_ctx))])) for _ in range(B)]
+    stage = ix.STAGE_FULL if rng.random() < 0.15 else ix.STAGE_CAUSAL
+    qwin = int(rng.integers(50, 2 * Tq)) if rng.random() < 0.25 else None
+    mode = int(rng.integers(0, 3))  # explicit workspace, the library's own scratch, no scratch
+    print(dict(D=D, H=H, G=G, Tq=Tq, kv_ctx=kv_ctx, W=W, B=B, phase=phase, tds=tds, stage=stage, qwin=qwin, mode=mode), flush=True)
+    gen = torch.Generator().manual_seed(13000 + n)
+    q = torch.randn(B, Tq, H, D, generator=gen).half().cuda().permute(0, 2, 1, 3)
+    o = torch.full((B, Tq, H, D), 777.0, dtype=torch.float16, device="cuda").permute(0, 2, 1, 3)
+    k = torch.randn(B, G, kv_ctx, D, generator=gen).half().cuda()
+    v = torch.randn(B, G, kv_ctx, D, generator=gen).half().cuda()
+    kw = dict(stage=stage, scale=D**-0.5, query_window=qwin)
+    ref = oracle(q, k, v, tds, phase, W, 1, **kw)
+    if mode == 0:
+        kw["workspace"] = torch.empty(max(fa2.workspace_bytes(B, H, G, Tq, D), 16), dtype=torch.uint8, device="cuda")
+    elif mode == 2:
+        kw["workspace"] = False
+    fa2.flash_attention(q, k, v, o, i32(tds), u8(phase), W, 1, **kw)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(got[b], ref[b], what=f"case {n} slot {b}")
+        else:
+            assert (got[b] == 777.0).all(), f"case {n}: off-phase slot {b} was written"

@@ -315,7 +315,7 @@ def test_random_launch_outside_the_tuned_shapes(gpu_device, n):
             assert (got[b] == sentinel).all(), f"case {n}: off-phase slot {b} was written"
 
 
-N_WORK_CASES = 16
+N_WORK_CASES = 40
 
 
 @pytest.mark.parametrize("n", range(N_WORK_CASES))

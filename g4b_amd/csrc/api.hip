@@ -105,18 +105,27 @@ bool prefill_pair_split(int H, int G, int Tq, int D) {
     const int tokb = bm / R, nq = (Tq + tokb - 1) / tokb;
     return (int64_t)nq * G * 2 > kPrefillFillWorkgroups && (int64_t)((nq + 1) / 2) * G * 2 <= kPrefillFillWorkgroups;
 }
+// One (slot, key split) pair of a prefill-shaped launch: its rows in the cache's 16-bit type, normalised by the split's
+// own sum, then (reference, sum) per row in fp32.
+uint64_t prefill_partial_bytes(int H, int Tq, int D) { return (uint64_t)H * (uint64_t)Tq * ((uint64_t)D * 2 + 2 * sizeof(float)); }
+float* prefill_partial_sums(void* workspace, int slots, int H, int Tq, int D) {
+    return reinterpret_cast<float*>(static_cast<char*>(workspace) + (uint64_t)slots * H * Tq * D * 2);
+}
 int prefill_split_slots(int H, int G, int Tq, int D) {
     const int R = H / G, bm = prefill_rows_per_workgroup(D);
     if (R < 1 || bm % R) return 0;
     const int tokb = bm / R;
     const int nq = (Tq + tokb - 1) / tokb;
     const int64_t per_slot = (int64_t)(prefill_pair_split(H, G, Tq, D) ? (nq + 1) / 2 : nq) * G;  // workgroups one slot brings
-    const int64_t slots = kPrefillFillWorkgroups / per_slot;
+    int64_t slots = kPrefillFillWorkgroups / per_slot;
+    // one query tile per workgroup and more than half of the units taken: under the causal mask the tiles' work grows
+    // linearly, so the launch takes as long as its last tile while the chip is half idle; two spans per tile halve that
+    if (slots < 2 && per_slot <= kPrefillFillWorkgroups && !prefill_pair_split(H, G, Tq, D)) slots = 2;
     if (slots < 2) return 0;
     return (int)(slots < kPrefillMaxSplitSlots ? slots : kPrefillMaxSplitSlots);
 }
 uint64_t prefill_workspace_bytes(int H, int G, int Tq, int D) {
-    return (uint64_t)prefill_split_slots(H, G, Tq, D) * (uint64_t)H * (uint64_t)Tq * (uint64_t)(D + 2) * sizeof(float);
+    return (uint64_t)prefill_split_slots(H, G, Tq, D) * prefill_partial_bytes(H, Tq, D);
 }
 
 }  // namespace
@@ -292,7 +301,7 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
             p.split_slots = prefill_split_slots(a->H, a->G, a->Tq, a->D);
             p.pair_split = prefill_pair_split(a->H, a->G, a->Tq, a->D) ? 1 : 0;
             p.part_o = static_cast<float*>(a->workspace);
-            p.part_ml = p.part_o + (uint64_t)p.split_slots * a->H * a->Tq * a->D;
+            p.part_ml = prefill_partial_sums(a->workspace, p.split_slots, a->H, a->Tq, a->D);
         }
         if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = a->D == 512 ? g4b::launch_attn_prefill_wide(p, a->kv_dtype, static_cast<hipStream_t>(stream))
@@ -339,7 +348,7 @@ MixedShape mixed_shape(int B, int H, int G, int D, int tq_pf, int tq_dec, bool p
     m.nw = (pair_path || !with_ws) ? 0 : nd * wpb;
     m.plan.nd_blocks = nd;
     m.plan.pair_path = pair_path ? 1 : 0;
-    m.pf_bytes = (uint64_t)m.split_slots * H * tq_pf * (uint64_t)(D + 2) * sizeof(float);
+    m.pf_bytes = (uint64_t)m.split_slots * prefill_partial_bytes(H, tq_pf, D);
     m.dec_bytes = m.nw ? decode_slots(B, G, m.nw) * (uint64_t)R * tq_dec * (uint64_t)(D + 2) * sizeof(float) : 0;
     return m;
 }
@@ -400,7 +409,7 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
         if (m.split_slots) {
             pp.split_slots = m.split_slots;
             pp.part_o = static_cast<float*>(a->workspace);
-            pp.part_ml = pp.part_o + (uint64_t)m.split_slots * a->H * a->Tq * a->D;
+            pp.part_ml = prefill_partial_sums(a->workspace, m.split_slots, a->H, a->Tq, a->D);
         }
         if (m.nw) {
             pd.NW = m.nw;

@@ -47,12 +47,12 @@ __global__ __launch_bounds__(256) void attn_mixed_kernel(const AttnParams pp, co
     }
 }
 
-template <int D>
+template <int D, class T>
 __global__ __launch_bounds__(256) void attn_mixed_combine(const AttnParams pp, const AttnParams pd, const MixedPlan mp) {
     __shared__ int sh_scan[8];
     __shared__ DecodeCombineSmem<D> sm;
     if ((int)blockIdx.x < mp.combine_pf) {
-        prefill_combine_body<D>(pp, blockIdx.x, sh_scan);
+        prefill_combine_body<D, T>(pp, blockIdx.x, sh_scan);
         return;
     }
     const int d = blockIdx.x - mp.combine_pf, rows = pd.R * pd.Tq;
@@ -72,7 +72,7 @@ static hipError_t launch_mixed_t(const AttnParams& pp, const AttnParams& pd, con
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if ((pp.kernel_mask & 2) && mp.combine_pf + mp.combine_dec > 0)
-        hipLaunchKernelGGL((attn_mixed_combine<D>), dim3(mp.combine_pf + mp.combine_dec), dim3(256), 0, stream, pp, pd, mp);
+        hipLaunchKernelGGL((attn_mixed_combine<D, T>), dim3(mp.combine_pf + mp.combine_dec), dim3(256), 0, stream, pp, pd, mp);
     return hipGetLastError();
 }
 

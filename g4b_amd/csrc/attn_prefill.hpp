@@ -493,7 +493,7 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     // 64 / (D/4) complete rows instead of touching 32 rows at 8 or 16 bytes each.
     const float l_tot = half_swap_sum(l_run);
     const bool partial = nsplit > 1 && !whole;
-    const float inv = partial ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;  // a key split's rows are normalised too: they are kept in 16 bits
     char* wbase = smem + wave * (32 * D * 4);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -520,9 +520,9 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
         const f4 v = *reinterpret_cast<const f4*>(wbase + row * (D * 4) + ((pc ^ (row & 15)) * 16));
         if (tr < Tq && (have_keys || !partial)) {  // a span without tiles of this query tile leaves (0, 0) in part_ml only
             if (partial) {
-                // un-normalised partial result of this key split: [pair][H][Tq][D] fp32
+                // this key split's result, normalised by its own sum, in the cache's type: [pair][H][Tq][D]
                 const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
-                *reinterpret_cast<f4*>(p.part_o + prow * D + pc * 4) = v;
+                store4(p.part_o, prow * D + pc * 4, T::dt, v);
             } else {
                 const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
                 // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2

@@ -288,7 +288,7 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
     // area per wave, free after the loop's last barrier), and stores 1 KiB row halves
     const float l_tot = half_swap_sum(l_run);
     const bool partial = nsplit > 1;
-    const float inv = partial ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;  // a key split's rows are normalised too: they are kept in 16 bits
     char* wbase = smem + wave * (32 * 256 * 4);
     if (partial && h2 == 0 && row_ok && (!QS || n32 < 16)) {
         const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hh)) * Tq + ti;
@@ -316,7 +316,7 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
             if (tr < Tq) {
                 if (partial) {
                     const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
-                    *reinterpret_cast<f4*>(p.part_o + prow * D + half * 256 + pc * 4) = v;
+                    store4(p.part_o, prow * D + half * 256 + pc * 4, T::dt, v);
                 } else {
                     const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
                     // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2

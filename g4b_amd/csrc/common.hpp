@@ -315,7 +315,8 @@ struct AttnParams {
     const int32_t* tds;
     const uint8_t* phase_arr;
     const int32_t* win_arr;  // optional per-slot window sizes
-    float* part_o;           // split partials: [slot][row][D] un-normalised fp32
+    float* part_o;           // split partials.  Decode: [slot][row][D] un-normalised fp32; prefill: [slot][row][D] in the
+                             // cache's 16-bit type, every row normalised by its own running sum
     float* part_ml;          // [slot][row][2] = (running max in log2 units, running sum)
     int64_t q_s[4], o_s[4];  // element strides of q and o ([B,H,Tq,D])
     int64_t k_sb, v_sb;      // batch strides of the caches (elements)

@@ -7,7 +7,7 @@ namespace g4b {
 // Merge the key splits of a prefill-shaped launch: a lane per four output columns of a row, PFC_ROWS rows per
 // workgroup, every load of a row independent of the others.
 constexpr int PFC_ROWS = 8;
-template <int D, int NS>
+template <int D, int NS, class T>
 G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, int tb, int nsplit) {
     constexpr int LPR = D / 4;      // lanes per row
     constexpr int RPP = 256 / LPR;  // rows per pass
@@ -32,7 +32,13 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
         for (int s = 0; s < NS; ++s) {
             const int64_t prow = ((int64_t)(a_idx * nsplit + min(s, nsplit - 1)) * p.H + h) * p.Tq + t;
             const f4 zero = {0.f, 0.f, 0.f, 0.f};
-            ov[s] = ls[s] > 0.f ? *reinterpret_cast<const f4*>(p.part_o + prow * D + d0) : zero;
+            if (ls[s] > 0.f) {
+                float x[4];
+                load_f32<4>(p.part_o, prow * D + d0, T::dt, x);
+                ov[s] = f4{x[0], x[1], x[2], x[3]};
+            } else {
+                ov[s] = zero;
+            }
         }
         float mref = -INFINITY;
 #pragma unroll
@@ -43,9 +49,9 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
 #pragma unroll
         for (int s = 0; s < NS; ++s)
             if (ls[s] > 0.f) {
-                const float w = fast_exp2(ms[s] - mref);
+                const float w = ls[s] * fast_exp2(ms[s] - mref);  // the split's rows were normalised by its sum
                 acc += ov[s] * w;
-                l += ls[s] * w;
+                l += w;
             }
         const float inv = l > 0.f ? 1.f / l : 0.f;
         const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)h * p.o_s[1] + (int64_t)t * p.o_s[2] + d0;
@@ -53,7 +59,7 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
     }
 }
 
-template <int D>
+template <int D, class T>
 G4B_DEV void prefill_combine_body(const AttnParams& p, const int bid, int* sh_scan) {
     const int tblocks = (p.Tq + PFC_ROWS - 1) / PFC_ROWS;
     const int a_idx = bid / (p.H * tblocks), h = (bid / tblocks) % p.H, tb = bid % tblocks;
@@ -61,16 +67,16 @@ G4B_DEV void prefill_combine_body(const AttnParams& p, const int bid, int* sh_sc
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);
     const int nsplit = prefill_splits(p.split_slots, n_active);
     if (b < 0 || nsplit == 1) return;
-    if (nsplit <= 2) prefill_combine_rows<D, 2>(p, a_idx, b, h, tb, nsplit);
-    else if (nsplit <= 4) prefill_combine_rows<D, 4>(p, a_idx, b, h, tb, nsplit);
-    else if (nsplit <= 8) prefill_combine_rows<D, 8>(p, a_idx, b, h, tb, nsplit);
-    else prefill_combine_rows<D, 16>(p, a_idx, b, h, tb, nsplit);
+    if (nsplit <= 2) prefill_combine_rows<D, 2, T>(p, a_idx, b, h, tb, nsplit);
+    else if (nsplit <= 4) prefill_combine_rows<D, 4, T>(p, a_idx, b, h, tb, nsplit);
+    else if (nsplit <= 8) prefill_combine_rows<D, 8, T>(p, a_idx, b, h, tb, nsplit);
+    else prefill_combine_rows<D, 16, T>(p, a_idx, b, h, tb, nsplit);
 }
 
-template <int D>
+template <int D, class T>
 __global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
     __shared__ int sh_scan[8];
-    prefill_combine_body<D>(p, blockIdx.x, sh_scan);
+    prefill_combine_body<D, T>(p, blockIdx.x, sh_scan);
 }
 
 // Workgroups the merge kernel of a split prefill-shaped launch needs (0 = the launch never splits).

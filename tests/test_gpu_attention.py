@@ -517,6 +517,33 @@ def test_prefill_3000_token_prompt_at_the_benchmark_head_shape(fa):
     assert_close(o.float().cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("case", ["from_scratch", "on_context", "two_active", "per_query_window", "bf16"])
+def test_head_dim_512_query_tiles_cut_into_two_key_spans(fa, case):
+    """Head dim 512 gives every workgroup one query tile; a slot whose tiles take more than half of the compute units
+    but not all of them (H/G = 16: 1500 tokens are 188 tiles of 8 tokens) has the keys of every tile cut into two
+    spans, so that the launch does not last as long as its heaviest tile with half of the chip idle.  With two slots in
+    phase the same launch runs unsplit."""
+    print(f"two key spans, D=512, {case}", flush=True)
+    H, G, Tq, D, kv_ctx = 16, 1, 1500, 512, 1800
+    B = 3 if case == "two_active" else 2
+    dtype = torch.bfloat16 if case == "bf16" else torch.float16
+    q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=len(case), dtype=dtype)
+    tds = {"from_scratch": [Tq, 5], "on_context": [kv_ctx + 300, 5], "two_active": [Tq, 1750, Tq + 7]}.get(case, [Tq + 130, 5])
+    phase = [1, 1, 0] if case == "two_active" else [1, 2]
+    kw = {"query_window": 300} if case == "per_query_window" else {}
+    assert fa.workspace_bytes(B, H, G, Tq, D) == 2 * H * Tq * (D * 2 + 8)
+    fa.flash_attention(q, k, v, o, i32(tds), u8(phase), kv_ctx, 1, scale=D**-0.5, **kw)
+    torch.cuda.synchronize()
+    ref = oracle(q, k, v, tds, phase, kv_ctx, 1, scale=D**-0.5, **kw)
+    got = o.float().cpu().numpy()
+    tol = dict(atol=ATOL_BF16, rtol=RTOL_BF16) if case == "bf16" else {}
+    for b in range(B):
+        if phase[b] == 1:
+            assert_close(got[b], ref[b], what=f"slot {b}", **tol)
+        else:
+            assert (got[b] == torch.tensor(777.0, dtype=dtype).float().item()).all()  # 776 in bf16
+
+
 @pytest.mark.parametrize("n_active", [5, 8, 9])
 def test_batch_of_prefill_chunks_one_query_tile_per_workgroup(fa, n_active):
     """Several slots with a 512-token chunk each (what the scheduler's prefill step looks like): too many for key splits,

@@ -79,11 +79,11 @@ def test_workspace_size_formula(native):
     # (workers + B*G) partial slots of rows x (D + 2) floats
     assert lib.g4b_attn_workspace_bytes(64, 8, 2, 1, 256, 0) == (nw + 128) * 4 * 258 * 4
     assert lib.g4b_attn_workspace_bytes(3, 8, 2, 2, 128, 10) == (10 + 6) * 8 * 130 * 4
-    # prefill-shaped: (slot, key split) pairs x H x Tq rows x (D + 2) floats when one slot brings fewer than 256
-    # workgroups (16 query tiles x 2 kv heads here -> 8 pairs), nothing when the shape fills the chip by itself
-    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 512, 256, 0) == 8 * 8 * 512 * 258 * 4
-    assert lib.g4b_attn_workspace_bytes(33, 8, 2, 512, 256, 0) == 8 * 8 * 512 * 258 * 4  # independent of B
-    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 2048, 256, 0) == 2 * 8 * 2048 * 258 * 4
+    # prefill-shaped: (slot, key split) pairs x H x Tq rows x (D 16-bit values + 2 floats) when one slot brings fewer
+    # than 256 workgroups (16 query tiles x 2 kv heads here -> 8 pairs), nothing when the shape fills the chip by itself
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 512, 256, 0) == 8 * 8 * 512 * (256 * 2 + 8)
+    assert lib.g4b_attn_workspace_bytes(33, 8, 2, 512, 256, 0) == 8 * 8 * 512 * (256 * 2 + 8)  # independent of B
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 2048, 256, 0) == 2 * 8 * 2048 * (256 * 2 + 8)
     assert lib.g4b_attn_workspace_bytes(1, 8, 2, 8192, 256, 0) == 0
 
 
@@ -263,15 +263,15 @@ def test_mixed_launch_is_validated_before_launching(native):
     with pytest.raises(NotImplementedError, match="head_dim"):
         flash_attention(q128, k128, k128, q128.clone(), tds, ph, T, PHASE_PREFILL, decode_q=torch.zeros(B, H, 1, 128, dtype=torch.float16),
                         decode_o=torch.zeros(B, H, 1, 128, dtype=torch.float16))
-    # sizing: the chunk's partials ((slot, split) pairs x H x t x (D + 2) floats, rounded up to 256 bytes) followed by the
+    # sizing: the chunk's partials ((slot, split) pairs x H x t x (D 16-bit values + 2 floats), rounded up to 256 bytes) followed by the
     # decode partials ((workers + B*G) x rows x (D + 2) floats).  64-token chunks bring 2 tiles x 2 kv heads = 4 workgroups
     # per slot; the default share-out leaves 256 - 112 = 144 units to the chunk -> 36 pairs, and the decode half gets the
     # remaining 112 workgroups of four workers.
     n = mixed_workspace_bytes(B, H, G, t, 1, D, T, T)
-    assert n == 36 * H * t * (D + 2) * 4 + (448 + B * G) * 4 * (D + 2) * 4
+    assert n == 36 * H * t * (D * 2 + 8) + (448 + B * G) * 4 * (D + 2) * 4
     # a short window takes the one-workgroup-per-pair decode path: no decode partials, 256 - B*G units for the chunk
     n_swa = mixed_workspace_bytes(B, H, G, t, 1, D, 512 + t - 1, 512)
-    assert n_swa == 63 * H * t * (D + 2) * 4
+    assert n_swa == 63 * H * t * (D * 2 + 8)
     assert mixed_workspace_bytes(B, H, G, t, 1, D, 512 + t - 1, 512, True) == n  # per-slot windows: streaming workers again
 
 

@@ -296,6 +296,7 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
         p.part_ml[prow * 2 + 1] = l_tot;
     }
     const int tokb_shift = __ffs(TOKB) - 1;  // TOKB = BM / R is a power of two
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // a row's head, token and offset are scalar arithmetic then
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -307,23 +308,35 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
                 const int pc = 8 * d8 + 2 * q4 + h2;
                 *reinterpret_cast<f4*>(wbase + n32 * 1024 + ((pc ^ (n32 & 15)) * 16)) = v;
             }
-#pragma unroll 4
-        for (int row = 0; row < WROWS; ++row) {  // with a split query the LDS rows 16..31 are copies of 0..15
-            const int pc = lane;  // 64 lanes x 16 bytes = 256 fp32 columns of one row
-            const int rr = wave * WROWS + row;
-            const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
-            const f4 v = *reinterpret_cast<const f4*>(wbase + row * 1024 + ((pc ^ (row & 15)) * 16));
-            if (tr < Tq) {
-                if (partial) {
-                    const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
-                    store4(p.part_o, prow * D + half * 256 + pc * 4, T::dt, v);
-                } else {
-                    const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
-                    // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2
-                    // (S = 8192 0.5 % faster, the 512-key sliding window 3.7 %; the same hint on the Q loads cost 1.3 .. 4 %)
-                    store4<true>(p.o, off + half * 256 + pc * 4, p.o_dt, v);
+        // Rows go eight at a time, their LDS reads first and in one block, with the split / final choice outside: row by
+        // row (read, wait, choose, convert, store) every row paid the LDS latency and a chain of branches by itself.
+        auto store_rows = [&](auto&& store_row) {
+#pragma unroll 1
+            for (int r0 = 0; r0 < WROWS; r0 += 8) {  // with a split query the LDS rows 16..31 are copies of 0..15
+                f4 v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)  // 64 lanes x 16 bytes = 256 fp32 columns of one row
+                    v[j] = *reinterpret_cast<const f4*>(wbase + (r0 + j) * 1024 + ((lane ^ ((r0 + j) & 15)) * 16));
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int rr = wave_u * WROWS + r0 + j;
+                    const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
+                    if (tr < Tq) store_row(hr, tr, v[j]);
                 }
             }
+        };
+        if (partial) {
+            store_rows([&](int hr, int tr, f4 v) {
+                const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
+                store4(p.part_o, prow * D + half * 256 + lane * 4, T::dt, v);
+            });
+        } else {
+            // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2
+            // (S = 8192 0.5 % faster, the 512-key sliding window 3.7 %; the same hint on the Q loads cost 1.3 .. 4 %)
+            store_rows([&](int hr, int tr, f4 v) {
+                const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
+                store4<true>(p.o, off + half * 256 + lane * 4, p.o_dt, v);
+            });
         }
     }
 }

@@ -512,43 +512,75 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     constexpr int LPR = D / 4;       // lanes that cover a row, 16 bytes of fp32 each
     constexpr int RPI = 64 / LPR;    // rows per store instruction
     const int tokb_shift = __ffs(TOKB) - 1;  // TOKB = 128 / R is a power of two
-    // The wave index as a scalar: with one row per instruction (D = 256) a row's head, token and 64-bit offset are then
-    // scalar arithmetic.  Rows go eight at a time, their LDS reads first and in one block, and the split / final choice
-    // sits outside the loop: a wave has its SIMD to itself here, and row by row -- read, wait, choose, convert, store --
-    // the 32 rows of a wave took 3.2 us without the stores themselves.
+    // Both destinations are rows of D elements at (head, token): the split's [pair][H][Tq][D] block in the cache's type,
+    // or o with the caller's strides and type.  A wave has its SIMD to itself here, so every instruction of this loop is
+    // four cycles of the workgroup's time: rows go eight at a time, their LDS reads first and in one block, the wave
+    // index is a scalar (a row's head, token and 64-bit offset are then scalar arithmetic), the type is chosen per
+    // batch and the rows of a batch are one offset plus a stride apart.  Row by row -- read, wait, compute the offset,
+    // choose the type, convert, store -- the 32 rows of a wave took 3.2 us before the stores themselves.
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    auto store_rows = [&](auto&& store_row) {
+    const int sub = lane / LPR, pc = lane % LPR;  // row inside an instruction's RPI rows, 16-byte piece of the row
+    void* dst;
+    int64_t head_stride, row_stride, base_off;
+    if (partial) {
+        dst = p.part_o;
+        head_stride = (int64_t)Tq * D;
+        row_stride = D;
+        base_off = ((int64_t)(a_idx * nsplit + split) * p.H + g * R) * head_stride;
+    } else {
+        dst = p.o;
+        head_stride = p.o_s[1];
+        row_stride = p.o_s[2];
+        base_off = (int64_t)b * p.o_s[0] + (int64_t)(g * R) * p.o_s[1];
+    }
+    auto store_rows = [&](auto nt, const int dt) {
+        constexpr bool NT = decltype(nt)::value;
 #pragma unroll 1
         for (int i0 = 0; i0 < 32 / RPI; i0 += 8) {
             f4 v[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const int row = (i0 + j) * RPI + lane / LPR, pc = lane % LPR;
+                const int row = (i0 + j) * RPI + sub;
                 v[j] = *reinterpret_cast<const f4*>(wbase + row * (D * 4) + ((pc ^ (row & 15)) * 16));
             }
+            const int rs = wave_u * 32 + i0 * RPI;  // first row of the batch
+            if (TOKB >= 8 * RPI) {
+                // the batch lies inside one head: consecutive tokens, one stride apart
+                const int hr = rs >> tokb_shift, tr0 = tok0 + (rs & (TOKB - 1));
+                const int64_t off0 = base_off + (int64_t)hr * head_stride + (int64_t)tr0 * row_stride;
+                const int64_t lane_off = (int64_t)sub * row_stride + pc * 4;
+                const int n_ok = Tq - tr0 - sub;  // token tr0 + j * RPI + sub is inside while j * RPI < n_ok
+                if (dt == DT_F32) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int rr = wave_u * 32 + (i0 + j) * RPI + lane / LPR;
-                const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
-                if (tr < Tq) store_row(hr, tr, lane % LPR, v[j]);
+                    for (int j = 0; j < 8; ++j)
+                        if (j * RPI < n_ok) store4<NT>(dst, off0 + (int64_t)(j * RPI) * row_stride + lane_off, DT_F32, v[j]);
+                } else if (dt == DT_F16) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (j * RPI < n_ok) store4<NT>(dst, off0 + (int64_t)(j * RPI) * row_stride + lane_off, DT_F16, v[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (j * RPI < n_ok) store4<NT>(dst, off0 + (int64_t)(j * RPI) * row_stride + lane_off, DT_BF16, v[j]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int rr = rs + j * RPI + sub;
+                    const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
+                    if (tr < Tq) store4<NT>(dst, base_off + (int64_t)hr * head_stride + (int64_t)tr * row_stride + pc * 4, dt, v[j]);
+                }
             }
         }
     };
     if (partial) {
-        if (have_keys) {  // a span without tiles of this query tile leaves (0, 0) in part_ml only
-            // this key split's result, normalised by its own sum, in the cache's type: [pair][H][Tq][D]
-            store_rows([&](int hr, int tr, int pc, f4 v) {
-                const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
-                store4(p.part_o, prow * D + pc * 4, T::dt, v);
-            });
-        }
+        // this key split's result, normalised by its own sum; a span without tiles of this query tile leaves (0, 0) in
+        // part_ml only
+        if (have_keys) store_rows(std::false_type{}, T::dt);
     } else {
         // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2
         // (S = 8192 0.5 % faster, the 512-key sliding window 3.7 %; the same hint on the Q loads cost 1.3 .. 4 %)
-        store_rows([&](int hr, int tr, int pc, f4 v) {
-            const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
-            store4<true>(p.o, off + pc * 4, p.o_dt, v);
-        });
+        store_rows(std::true_type{}, p.o_dt);
     }
     }
 }

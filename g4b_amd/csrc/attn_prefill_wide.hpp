@@ -297,6 +297,21 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
     }
     const int tokb_shift = __ffs(TOKB) - 1;  // TOKB = BM / R is a power of two
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // a row's head, token and offset are scalar arithmetic then
+    // both destinations are rows of D elements at (head, token): the split's [pair][H][Tq][D] block in the cache's type,
+    // or o with the caller's strides and type
+    void* dst;
+    int64_t head_stride, row_stride, base_off;
+    if (partial) {
+        dst = p.part_o;
+        head_stride = (int64_t)Tq * D;
+        row_stride = D;
+        base_off = ((int64_t)(a_idx * nsplit + split) * p.H + g * R) * head_stride;
+    } else {
+        dst = p.o;
+        head_stride = p.o_s[1];
+        row_stride = p.o_s[2];
+        base_off = (int64_t)b * p.o_s[0] + (int64_t)(g * R) * p.o_s[1];
+    }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -308,36 +323,52 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
                 const int pc = 8 * d8 + 2 * q4 + h2;
                 *reinterpret_cast<f4*>(wbase + n32 * 1024 + ((pc ^ (n32 & 15)) * 16)) = v;
             }
-        // Rows go eight at a time, their LDS reads first and in one block, with the split / final choice outside: row by
-        // row (read, wait, choose, convert, store) every row paid the LDS latency and a chain of branches by itself.
-        auto store_rows = [&](auto&& store_row) {
+        // Rows go eight at a time, their LDS reads first and in one block; the type is chosen per batch and the rows of
+        // a batch are one scalar offset plus a stride apart (a wave has its SIMD to itself here: row by row -- read,
+        // wait, compute the offset, choose the type, convert, store -- every row paid the LDS latency and some thirty
+        // instructions by itself).
+        auto store_rows = [&](auto nt, const int dt) {
+            constexpr bool NT = decltype(nt)::value;
 #pragma unroll 1
             for (int r0 = 0; r0 < WROWS; r0 += 8) {  // with a split query the LDS rows 16..31 are copies of 0..15
                 f4 v[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j)  // 64 lanes x 16 bytes = 256 fp32 columns of one row
                     v[j] = *reinterpret_cast<const f4*>(wbase + (r0 + j) * 1024 + ((lane ^ ((r0 + j) & 15)) * 16));
+                const int rs = wave_u * WROWS + r0;  // first row of the batch
+                if (TOKB >= 8) {
+                    // the batch lies inside one head: consecutive tokens, one stride apart
+                    const int hr = rs >> tokb_shift, tr0 = tok0 + (rs & (TOKB - 1));
+                    const int64_t off0 = base_off + (int64_t)hr * head_stride + (int64_t)tr0 * row_stride + half * 256;
+                    const int n_ok = Tq - tr0;
+                    if (dt == DT_F32) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int rr = wave_u * WROWS + r0 + j;
-                    const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
-                    if (tr < Tq) store_row(hr, tr, v[j]);
+                        for (int j = 0; j < 8; ++j)
+                            if (j < n_ok) store4<NT>(dst, off0 + (int64_t)j * row_stride + lane * 4, DT_F32, v[j]);
+                    } else if (dt == DT_F16) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            if (j < n_ok) store4<NT>(dst, off0 + (int64_t)j * row_stride + lane * 4, DT_F16, v[j]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            if (j < n_ok) store4<NT>(dst, off0 + (int64_t)j * row_stride + lane * 4, DT_BF16, v[j]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int rr = rs + j;
+                        const int hr = rr >> tokb_shift, tr = tok0 + (rr & (TOKB - 1));
+                        if (tr < Tq)
+                            store4<NT>(dst, base_off + (int64_t)hr * head_stride + (int64_t)tr * row_stride + half * 256 + lane * 4, dt, v[j]);
+                    }
                 }
             }
         };
-        if (partial) {
-            store_rows([&](int hr, int tr, f4 v) {
-                const int64_t prow = ((int64_t)(a_idx * nsplit + split) * p.H + (g * R + hr)) * Tq + tr;
-                store4(p.part_o, prow * D + half * 256 + lane * 4, T::dt, v);
-            });
-        } else {
-            // written once and not read here again: non-temporal, so that the rows do not displace K/V tiles in L2
-            // (S = 8192 0.5 % faster, the 512-key sliding window 3.7 %; the same hint on the Q loads cost 1.3 .. 4 %)
-            store_rows([&](int hr, int tr, f4 v) {
-                const int64_t off = (int64_t)b * p.o_s[0] + (int64_t)(g * R + hr) * p.o_s[1] + (int64_t)tr * p.o_s[2];
-                store4<true>(p.o, off + half * 256 + lane * 4, p.o_dt, v);
-            });
-        }
+        // written once and not read here again: o goes out non-temporal, so that the rows do not displace K/V tiles in
+        // L2 (S = 8192 0.5 % faster, the 512-key sliding window 3.7 %; the same hint on the Q loads cost 1.3 .. 4 %)
+        if (partial) store_rows(std::false_type{}, T::dt);
+        else store_rows(std::true_type{}, p.o_dt);
     }
 }
 

@@ -27,9 +27,23 @@ namespace g4b {
 
 constexpr int DEC_TILE = 32;  // keys per wave iteration
 
-G4B_DEV int slot_tiles(const AttnParams& p, int b) {
-    SlotInfo s = slot_info(p, b);
-    return (s.window - s.klo + DEC_TILE - 1) / DEC_TILE;
+G4B_DEV int slot_tiles(const SlotInfo& s) { return (s.window - s.klo + DEC_TILE - 1) / DEC_TILE; }
+G4B_DEV int slot_tiles(const AttnParams& p, int b) { return slot_tiles(slot_info(p, b)); }
+// What lane `src` of the wave holds, for every lane (src is the same in all of them).
+G4B_DEV SlotInfo slot_info_of_lane(const SlotInfo& s, int src) {
+    SlotInfo r;
+    r.window = __shfl(s.window, src);
+    r.ring_start = __shfl(s.ring_start, src);
+    r.qb = __shfl(s.qb, src);
+    r.klo = __shfl(s.klo, src);
+    r.active = __shfl((int)s.active, src) != 0;
+    return r;
+}
+// floor(a * b / c) for a * b below 2^63; in 32 bits when the caller knows that a * b fits (`small`, the same in every
+// lane): a 64-bit division is some 150 instructions, and a decode worker makes two of them before its first load.
+G4B_DEV int64_t muldiv(int64_t a, int64_t b, int64_t c, bool small) {
+    if (small) return (int64_t)((uint32_t)a * (uint32_t)b / (uint32_t)c);
+    return a * b / c;
 }
 
 template <int CL>
@@ -59,8 +73,8 @@ G4B_DEV float pick(const f4& c, int e, int cls) {
 // QS: the query is wider than the cache type and enters the first product as two operands (rounded value, rounding
 // error), so the scores see the unrounded query.
 template <int D, int CL, class T, int DH, bool QS>
-G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, int t1, int tlb, float* xch,
-                            float* lds_part = nullptr) {
+G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int bb, int g, int t0, int t1, int tlb,
+                            float* xch, float* lds_part = nullptr) {
     constexpr int DL = D / DH;         // columns this wave owns
     constexpr int E = 4 / CL;          // scores a lane keeps per 16-row MFMA tile
     constexpr int KT = 16 / CL;        // keys per MFMA tile
@@ -77,7 +91,6 @@ G4B_DEV void decode_segment(const AttnParams& p, int w, int bb, int g, int t0, i
     const int G = p.G, Tq = p.Tq;
     const int NR = p.R * Tq;
 
-    const SlotInfo si = slot_info(p, bb);
     const int KV_CTX = p.KV_CTX;
     const char* kbase =
         static_cast<const char*>(p.k) + ((int64_t)bb * p.k_sb + (int64_t)g * KV_CTX * D + hv * DL) * 2;
@@ -280,10 +293,11 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
         // no workspace: worker w owns the whole pair w
         if (w >= B * G) return;
         const int bb = w / G, g = w % G;
-        const int tlb = slot_tiles(p, bb);
+        const SlotInfo si = slot_info(p, bb);
+        const int tlb = slot_tiles(si);
         if (tlb > 0) {
-            decode_segment<D, CL, T, DH, QS>(p, w, bb, g, 0, tlb, tlb, xch);
-        } else if (slot_info(p, bb).active && (DH == 1 || threadIdx.x < 64)) {  // one wave of the worker
+            decode_segment<D, CL, T, DH, QS>(p, si, w, bb, g, 0, tlb, tlb, xch);
+        } else if (si.active && (DH == 1 || threadIdx.x < 64)) {  // one wave of the worker
             // in-phase slot without any visible key: defined as zeros (no merge kernel runs on this path)
             const int NR = p.R * p.Tq;
             for (int idx = lane; idx < NR * (D / 4); idx += 64) {
@@ -297,21 +311,31 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
     }
 
     // ---- flat tile list: total, then this worker's range ------------------------------------
-    int total = 0;
+    // lane l keeps what it read of slot l (the first 64 slots) for the second pass and for the segments
+    int total = 0, tl_first = 0;
+    SlotInfo si_first = {};
     for (int b0 = 0; b0 < B; b0 += 64) {
-        int b = b0 + lane;
-        total += (b < B) ? G * slot_tiles(p, b) : 0;
+        const int b = b0 + lane;
+        int tl = 0;
+        if (b < B) {
+            const SlotInfo s = slot_info(p, b);
+            tl = slot_tiles(s);
+            if (b0 == 0) si_first = s;
+        }
+        if (b0 == 0) tl_first = tl;
+        total += G * tl;
     }
     total = wave_sum_i(total);
     const int nw = min(p.NW, total);  // never more workers than tiles: every worker below nw owns >= 1 tile
     if (w >= nw) return;
-    const int64_t ws = (int64_t)w * total / nw;
-    const int64_t we = (int64_t)(w + 1) * total / nw;
+    const bool small = (uint64_t)total * (uint64_t)nw < ((uint64_t)1 << 32);
+    const int64_t ws = muldiv(w, total, nw, small);
+    const int64_t we = muldiv(w + 1, total, nw, small);
 
     int carry = 0;
     for (int b0 = 0; b0 < B; b0 += 64) {
         const int bl = b0 + lane;
-        const int tl = (bl < B) ? slot_tiles(p, bl) : 0;
+        const int tl = b0 == 0 ? tl_first : ((bl < B) ? slot_tiles(p, bl) : 0);
         const int cnt = G * tl;
         const int incl = wave_incl_scan_i(cnt, lane);
         const int excl = carry + incl - cnt;
@@ -323,11 +347,12 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
             const int bb = b0 + src;
             const int ex = __shfl(excl, src);
             const int tlb = __shfl(tl, src);
+            const SlotInfo si = b0 == 0 ? slot_info_of_lane(si_first, src) : slot_info(p, bb);
             for (int g = 0; g < G; ++g) {
                 const int64_t fs = (int64_t)ex + (int64_t)g * tlb;
                 const int t0 = (int)(max(ws, fs) - fs);
                 const int t1 = (int)(min(we, fs + tlb) - fs);
-                if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, w, bb, g, t0, t1, tlb, xch);
+                if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, si, w, bb, g, t0, t1, tlb, xch);
             }
         }
         carry += __shfl(incl, 63);
@@ -356,11 +381,11 @@ G4B_DEV void decode_pair_body(const AttnParams& p, int pair, float* pair_smem) {
     const SlotInfo si = slot_info(p, bb);
     if (!si.active) return;
     const int NR = p.R * p.Tq;
-    const int tl = slot_tiles(p, bb);
+    const int tl = slot_tiles(si);
     float* mine = pair_smem + wave * BLK;
     const int t0 = wave * tl / DEC_PAIR_WAVES, t1 = (wave + 1) * tl / DEC_PAIR_WAVES;
     if (t1 > t0) {
-        decode_segment<D, CL, T, 1, QS>(p, 0, bb, g, t0, t1, tl, nullptr, mine);
+        decode_segment<D, CL, T, 1, QS>(p, si, 0, bb, g, t0, t1, tl, nullptr, mine);
     } else if ((tid & 63) < 16) {
         mine[16 * D + (tid & 63) * 2] = -INFINITY;  // this wave brought no keys
         mine[16 * D + (tid & 63) * 2 + 1] = 0.f;
@@ -419,18 +444,24 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
 
     // flat start of this pair and total tile count (same arithmetic as the workers), computed by every wave
     int before = 0, total = 0;
+    SlotInfo si_first = {};  // lane l keeps what it read of slot l (the first 64 slots)
     for (int b0 = 0; b0 < B; b0 += 64) {
         const int x = b0 + lane;
-        const int c = (x < B) ? G * slot_tiles(p, x) : 0;
+        int c = 0;
+        if (x < B) {
+            const SlotInfo s = slot_info(p, x);
+            c = G * slot_tiles(s);
+            if (b0 == 0) si_first = s;
+        }
         total += c;
         before += (x < b) ? c : 0;
     }
     total = wave_sum_i(total);
     before = wave_sum_i(before);
 
-    const SlotInfo si = slot_info(p, b);
+    const SlotInfo si = b < 64 ? slot_info_of_lane(si_first, b) : slot_info(p, b);
     if (!si.active) return;
-    const int tl = slot_tiles(p, b);
+    const int tl = slot_tiles(si);
     const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] + (int64_t)(row % p.Tq) * p.o_s[2];
     if (tl == 0) {
         // in-phase slot without any visible key: defined as zeros
@@ -441,8 +472,15 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
     const int nw = min(p.NW, total);
     const int64_t fs = (int64_t)before + (int64_t)g * tl;
     // worker that owns flat tile x: the largest w with floor(w * total / nw) <= x
-    const int w0 = (int)(((fs + 1) * nw - 1) / total);
-    const int w1 = (int)(((fs + tl) * nw - 1) / total);
+    const bool small = (uint64_t)total * (uint64_t)nw < ((uint64_t)1 << 32);  // (fs + tl) * nw <= total * nw
+    int w0, w1;
+    if (small) {
+        w0 = (int)(((uint32_t)(fs + 1) * (uint32_t)nw - 1u) / (uint32_t)total);
+        w1 = (int)(((uint32_t)(fs + tl) * (uint32_t)nw - 1u) / (uint32_t)total);
+    } else {
+        w0 = (int)(((fs + 1) * nw - 1) / total);
+        w1 = (int)(((fs + tl) * nw - 1) / total);
+    }
     if (w0 == w1) return;  // a single worker owned the pair and wrote the output itself
 
     // partial of worker w for this pair and row: slot w + pair

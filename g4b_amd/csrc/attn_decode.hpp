@@ -211,8 +211,7 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
         float mx = sc[0];
 #pragma unroll
         for (int s = 1; s < 8; ++s) mx = fmaxf(mx, sc[s]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = half_swap_max(row_swap_max(mx));  // over the lanes l, l ^ 16, l ^ 32, l ^ 48 that share a query row
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = fast_exp2(m_run - m_safe);
@@ -240,8 +239,7 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
     }
 
     // ---- epilogue -----------------------------------------------------------------
-    float l_tot = l_run + __shfl_xor(l_run, 16);
-    l_tot += __shfl_xor(l_tot, 32);
+    const float l_tot = half_swap_sum(row_swap_sum(l_run));
     const bool whole = (t0 == 0 && t1 == tlb) && lds_part == nullptr;
     if (row_ok) {
         if (whole) {

@@ -223,18 +223,43 @@ G4B_DEV float dpp_f(float x) {
 G4B_DEV float quad_xor1(float x) { return dpp_f<0xB1>(x); }  // quad_perm [1,0,3,2]
 G4B_DEV float quad_xor2(float x) { return dpp_f<0x4E>(x); }  // quad_perm [2,3,0,1]
 
+// Sum over the wave, in every lane, and inclusive prefix sum over the lanes.  Both stay in the vector ALU (DPP inside
+// the rows of 16 lanes, then lane reads / row broadcasts across them): six dependent shuffles through the LDS crossbar
+// were 0.3 us each at the head of every decode worker and merge workgroup.
+template <int CTRL, int ROW_MASK = 0xf>
+G4B_DEV int dpp_i0(int x) {  // lanes the pattern leaves without a source, or masks out, read 0
+    return __builtin_amdgcn_update_dpp(0, x, CTRL, ROW_MASK, 0xf, false);
+}
 G4B_DEV int wave_sum_i(int v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    v += dpp_i0<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_i0<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_i0<0x141>(v);  // row_half_mirror
+    v += dpp_i0<0x140>(v);  // row_mirror: every lane holds its row's sum
+    return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+           __builtin_amdgcn_readlane(v, 48);
+}
+G4B_DEV int wave_incl_scan_i(int v, int /*lane*/) {
+    v += dpp_i0<0x111>(v);       // row_shr:1
+    v += dpp_i0<0x112>(v);       // row_shr:2
+    v += dpp_i0<0x114>(v);       // row_shr:4
+    v += dpp_i0<0x118>(v);       // row_shr:8: inclusive inside every row
+    v += dpp_i0<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_i0<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
     return v;
 }
-G4B_DEV int wave_incl_scan_i(int v, int lane) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        int t = __shfl_up(v, o);
-        if (lane >= o) v += t;
-    }
-    return v;
+// max / sum over the lanes l, l ^ 16: v_permlane16_swap exchanges the odd rows of its first operand with the even rows
+// of its second, so that of the two results one is the lane's own value and the other its partner's.
+G4B_DEV float row_swap_max(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    const u2 r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+G4B_DEV float row_swap_sum(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    const u2 r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
 }
 
 G4B_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -483,24 +483,16 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
 
     // partial of worker w for this pair and row: slot w + pair
     auto ml_of = [&](int w) { return p.part_ml + (((int64_t)w + pair) * NR + row) * 2; };
-    // pass 1: the row's reference = largest reference any worker used (-inf marks a worker without keys for the row)
-    float mref = -INFINITY;
-    for (int w = w0 + tid; w <= w1; w += 256) mref = fmaxf(mref, ml_of(w)[0]);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mref = fmaxf(mref, __shfl_xor(mref, o));
-    if (lane == 0) sm_max[wave] = mref;
-    __syncthreads();
-    mref = fmaxf(fmaxf(sm_max[0], sm_max[1]), fmaxf(sm_max[2], sm_max[3]));
-    const float msafe = (mref == -INFINITY) ? 0.f : mref;
-
-    // pass 2: wave k takes workers w0 + k, w0 + k + 4, ...; a lane owns four output columns
+    // Wave k takes workers w0 + k, w0 + k + 4, ...; a lane owns four output columns.  Every wave sums its workers
+    // against a reference of its own (the largest one it has seen, -inf marks a worker without keys for the row), so
+    // that nothing waits for a first pass over all references; the four waves are merged through LDS at the end.
     constexpr int LPR = D / 4 < 64 ? D / 4 : 64;  // lanes that hold a row
     constexpr int NV = D / 4 / LPR;               // float4 pieces per lane: piece v covers columns (v*64 + lane)*4..+3
-    constexpr int UN = 8;
+    constexpr int UN = NV == 1 ? 16 : 8;          // workers whose loads are in flight together
     f4 acc[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) acc[v] = f4{0.f, 0.f, 0.f, 0.f};
-    float l = 0.f;
+    float l = 0.f, ref = -INFINITY;
     for (int wb = w0 + wave; wb <= w1; wb += 4 * UN) {
         float wgt[UN], lw[UN];
         f4 ov[UN][NV];
@@ -515,11 +507,22 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
             for (int v = 0; v < NV; ++v)
                 ov[u][v] = (lane < LPR) ? *reinterpret_cast<const f4*>(po + (v * 64 + lane) * 4) : f4{0.f, 0.f, 0.f, 0.f};
         }
+        float bm = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (wb + 4 * u <= w1) bm = fmaxf(bm, wgt[u]);
+        if (bm > ref) {  // the same in every lane
+            const float a = fast_exp2(ref - bm);  // 0 while ref is -inf
+#pragma unroll
+            for (int v = 0; v < NV; ++v) acc[v] = acc[v] * a;
+            l *= a;
+            ref = bm;
+        }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const bool live = (wb + 4 * u <= w1) && (wgt[u] != -INFINITY);
-            const float e = live ? fast_exp2(wgt[u] - msafe) : 0.f;
             if (live) {
+                const float e = fast_exp2(wgt[u] - ref);
 #pragma unroll
                 for (int v = 0; v < NV; ++v) acc[v] += ov[u][v] * e;
                 l += lw[u] * e;
@@ -530,11 +533,21 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
 #pragma unroll
         for (int v = 0; v < NV; ++v) sm_acc[wave][v * 64 + lane] = acc[v];
     }
-    if (lane == 0) sm_l[wave] = l;
+    if (lane == 0) {
+        sm_l[wave] = l;
+        sm_max[wave] = ref;
+    }
     __syncthreads();
     if (tid < D / 4) {
-        const f4 r = sm_acc[0][tid] + sm_acc[1][tid] + sm_acc[2][tid] + sm_acc[3][tid];
-        const float lt = sm_l[0] + sm_l[1] + sm_l[2] + sm_l[3];
+        const float mref = fmaxf(fmaxf(sm_max[0], sm_max[1]), fmaxf(sm_max[2], sm_max[3]));
+        f4 r = {0.f, 0.f, 0.f, 0.f};
+        float lt = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float e = sm_max[k] == -INFINITY ? 0.f : fast_exp2(sm_max[k] - mref);
+            r += sm_acc[k][tid] * e;
+            lt += sm_l[k] * e;
+        }
         const float inv = lt > 0.f ? 1.f / lt : 0.f;
         store4(p.o, ooff + tid * 4, p.o_dt, r * inv);
     }

@@ -29,14 +29,14 @@ constexpr int DEC_TILE = 32;  // keys per wave iteration
 
 G4B_DEV int slot_tiles(const SlotInfo& s) { return (s.window - s.klo + DEC_TILE - 1) / DEC_TILE; }
 G4B_DEV int slot_tiles(const AttnParams& p, int b) { return slot_tiles(slot_info(p, b)); }
-// What lane `src` of the wave holds, for every lane (src is the same in all of them).
+// What lane `src` of the wave holds, for every lane (src must be the same in all of them: a lane read, not a shuffle).
 G4B_DEV SlotInfo slot_info_of_lane(const SlotInfo& s, int src) {
     SlotInfo r;
-    r.window = __shfl(s.window, src);
-    r.ring_start = __shfl(s.ring_start, src);
-    r.qb = __shfl(s.qb, src);
-    r.klo = __shfl(s.klo, src);
-    r.active = __shfl((int)s.active, src) != 0;
+    r.window = __builtin_amdgcn_readlane(s.window, src);
+    r.ring_start = __builtin_amdgcn_readlane(s.ring_start, src);
+    r.qb = __builtin_amdgcn_readlane(s.qb, src);
+    r.klo = __builtin_amdgcn_readlane(s.klo, src);
+    r.active = __builtin_amdgcn_readlane((int)s.active, src) != 0;
     return r;
 }
 // floor(a * b / c) for a * b below 2^63; in 32 bits when the caller knows that a * b fits (`small`, the same in every
@@ -343,8 +343,8 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
             const int src = __builtin_ctzll(mask);
             mask &= mask - 1;
             const int bb = b0 + src;
-            const int ex = __shfl(excl, src);
-            const int tlb = __shfl(tl, src);
+            const int ex = __builtin_amdgcn_readlane(excl, src);
+            const int tlb = __builtin_amdgcn_readlane(tl, src);
             const SlotInfo si = b0 == 0 ? slot_info_of_lane(si_first, src) : slot_info(p, bb);
             for (int g = 0; g < G; ++g) {
                 const int64_t fs = (int64_t)ex + (int64_t)g * tlb;
@@ -353,7 +353,7 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
                 if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, si, w, bb, g, t0, t1, tlb, xch);
             }
         }
-        carry += __shfl(incl, 63);
+        carry += __builtin_amdgcn_readlane(incl, 63);
         if ((int64_t)carry >= we) break;
     }
 }

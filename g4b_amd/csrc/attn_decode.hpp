@@ -29,16 +29,6 @@ constexpr int DEC_TILE = 32;  // keys per wave iteration
 
 G4B_DEV int slot_tiles(const SlotInfo& s) { return (s.window - s.klo + DEC_TILE - 1) / DEC_TILE; }
 G4B_DEV int slot_tiles(const AttnParams& p, int b) { return slot_tiles(slot_info(p, b)); }
-// What lane `src` of the wave holds, for every lane (src must be the same in all of them: a lane read, not a shuffle).
-G4B_DEV SlotInfo slot_info_of_lane(const SlotInfo& s, int src) {
-    SlotInfo r;
-    r.window = __builtin_amdgcn_readlane(s.window, src);
-    r.ring_start = __builtin_amdgcn_readlane(s.ring_start, src);
-    r.qb = __builtin_amdgcn_readlane(s.qb, src);
-    r.klo = __builtin_amdgcn_readlane(s.klo, src);
-    r.active = __builtin_amdgcn_readlane((int)s.active, src) != 0;
-    return r;
-}
 // floor(a * b / c) for a * b below 2^63; in 32 bits when the caller knows that a * b fits (`small`, the same in every
 // lane): a 64-bit division is some 150 instructions, and a decode worker makes two of them before its first load.
 G4B_DEV int64_t muldiv(int64_t a, int64_t b, int64_t c, bool small) {

@@ -74,8 +74,18 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     const int TOKB = PF_BM / R;
     // The work list is built from the slots that are in phase, so a launch with few of them (one prefill chunk in a
     // batch of decoding slots) can split every item's keys over several workgroups and still fill the chip.
+    // A launch of up to 64 slots reads every slot's data in one round, lane l slot l: the in-phase slots are a ballot
+    // away, and the slot this workgroup works on is a lane read instead of a second round of loads behind the first.
     int n_active;
-    nth_active_slot(p, -1, n_active, sh_scan);
+    SlotInfo mine = {};
+    unsigned long long in_phase = 0;
+    if (p.B <= 64) {
+        if (lane < p.B) mine = slot_info(p, lane);
+        in_phase = __ballot(mine.active);
+        n_active = __popcll(in_phase);
+    } else {
+        nth_active_slot(p, -1, n_active, sh_scan);
+    }
     if (n_active == 0) return;
     const int nsplit = prefill_splits(p.part_o ? p.split_slots : 1, n_active);
     const int nq_tiles = (Tq + TOKB - 1) / TOKB;
@@ -95,9 +105,16 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
     const int qtile_second = near_pair ? 2 * rank : rank;
     const int n_items = (ipw == 2 && qtile_second != qtile_first) ? 2 : 1;
     const int split = head % nsplit, g = (head / nsplit) % p.G, a_idx = head / (nsplit * p.G);
-    const int b = nth_active_slot(p, a_idx, n_active, sh_scan);  // workgroup-uniform
-
-    const SlotInfo si = slot_info(p, b);
+    int b;  // workgroup-uniform
+    SlotInfo si;
+    if (p.B <= 64) {
+        const unsigned long long hit = __ballot(mine.active && __popcll(in_phase & ((1ull << lane) - 1ull)) == a_idx);
+        b = __ffsll((long long)hit) - 1;  // a_idx < n_active: the grid map hands out no other
+        si = slot_info_of_lane(mine, b);
+    } else {
+        b = nth_active_slot(p, a_idx, n_active, sh_scan);
+        si = slot_info(p, b);
+    }
 
     // Key splits: the key tiles of the workgroup's query tiles -- the first tile's, then the second's -- are one list
     // that is cut into nsplit equal spans; this workgroup owns span `split` (tiles [span0, span1) of the list).

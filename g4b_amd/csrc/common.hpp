@@ -382,6 +382,16 @@ G4B_DEV SlotInfo slot_info(const AttnParams& p, int b) {
     return s;
 }
 
+// What lane `src` of the wave holds, for every lane (src must be the same in all of them: a lane read, not a shuffle).
+G4B_DEV SlotInfo slot_info_of_lane(const SlotInfo& s, int src) {
+    SlotInfo r;
+    r.window = __builtin_amdgcn_readlane(s.window, src);
+    r.ring_start = __builtin_amdgcn_readlane(s.ring_start, src);
+    r.qb = __builtin_amdgcn_readlane(s.qb, src);
+    r.klo = __builtin_amdgcn_readlane(s.klo, src);
+    r.active = __builtin_amdgcn_readlane((int)s.active, src) != 0;
+    return r;
+}
 // Number of slots whose phase matches the launch (n_active) and the index of the a-th of them (-1 when a is out of
 // range).  Every thread of a workgroup of NWAVES waves must call it; sh is workgroup-shared scratch of at least
 // NWAVES + 1 ints.  Call it with a < 0 to count only.

@@ -16,7 +16,7 @@ static hipError_t launch_prefill_ps(const AttnParams& p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_kernel<D, T, QS, PS>), grid, dim3(256), smem, stream, p);
     if (slots > 1 && (p.kernel_mask & 2))
-        hipLaunchKernelGGL((attn_prefill_combine<D, T>), dim3(prefill_combine_grid(p)), dim3(256), 0, stream, p);
+        launch_prefill_combine<D, T>(p, slots, stream);
     return hipGetLastError();
 }
 

@@ -13,7 +13,7 @@ static hipError_t launch_prefill_wide_t(const AttnParams& p, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (p.kernel_mask & 1) G4B_LAUNCH_DOMINANT((attn_prefill_wide_kernel<T, QS>), dim3(blocks), dim3(256), PW_SMEM, stream, p);
     if (slots > 1 && (p.kernel_mask & 2))
-        hipLaunchKernelGGL((attn_prefill_combine<PW_D, T>), dim3(prefill_combine_grid(p)), dim3(256), 0, stream, p);
+        launch_prefill_combine<PW_D, T>(p, slots, stream);
     return hipGetLastError();
 }
 

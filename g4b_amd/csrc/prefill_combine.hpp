@@ -59,7 +59,19 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
     }
 }
 
-template <int D, class T>
+// Workgroups the merge kernel of a split prefill-shaped launch needs (0 = the launch never splits).
+inline int prefill_combine_grid_of(const AttnParams& p, int slots) {
+    if (slots <= 1) return 0;
+    const int items = p.B < slots / 2 ? p.B : slots / 2;  // more active slots than this are never split
+    return items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS);
+}
+inline int prefill_combine_grid(const AttnParams& p) { return prefill_combine_grid_of(p, p.part_o ? p.split_slots : 1); }
+
+// NSMAX: the most key splits the launch can have (its split_slots, which the host knows; the split count itself follows
+// the number of in-phase slots, which only the device knows).  The wide variants hold up to 16 partial rows per lane
+// and set the kernel's register count; a launch that cannot need them takes a kernel without them, twice as many of
+// whose workgroups fit a compute unit (the merge of the S = 2048 launch ran its 2048 workgroups in two rounds).
+template <int D, class T, int NSMAX = 16>
 G4B_DEV void prefill_combine_body(const AttnParams& p, const int bid, int* sh_scan) {
     const int tblocks = (p.Tq + PFC_ROWS - 1) / PFC_ROWS;
     const int a_idx = bid / (p.H * tblocks), h = (bid / tblocks) % p.H, tb = bid % tblocks;
@@ -67,24 +79,32 @@ G4B_DEV void prefill_combine_body(const AttnParams& p, const int bid, int* sh_sc
     const int b = nth_active_slot(p, a_idx, n_active, sh_scan);
     const int nsplit = prefill_splits(p.split_slots, n_active);
     if (b < 0 || nsplit == 1) return;
-    if (nsplit <= 2) prefill_combine_rows<D, 2, T>(p, a_idx, b, h, tb, nsplit);
-    else if (nsplit <= 4) prefill_combine_rows<D, 4, T>(p, a_idx, b, h, tb, nsplit);
-    else if (nsplit <= 8) prefill_combine_rows<D, 8, T>(p, a_idx, b, h, tb, nsplit);
-    else prefill_combine_rows<D, 16, T>(p, a_idx, b, h, tb, nsplit);
+    if (nsplit <= 2) {
+        prefill_combine_rows<D, 2, T>(p, a_idx, b, h, tb, nsplit);
+    } else if constexpr (NSMAX >= 4) {
+        if (nsplit <= 4) {
+            prefill_combine_rows<D, 4, T>(p, a_idx, b, h, tb, nsplit);
+        } else if constexpr (NSMAX >= 8) {
+            if (nsplit <= 8) prefill_combine_rows<D, 8, T>(p, a_idx, b, h, tb, nsplit);
+            else if constexpr (NSMAX >= 16) prefill_combine_rows<D, 16, T>(p, a_idx, b, h, tb, nsplit);
+        }
+    }
 }
 
-template <int D, class T>
+template <int D, class T, int NSMAX>
 __global__ __launch_bounds__(256) void attn_prefill_combine(const AttnParams p) {
     __shared__ int sh_scan[8];
-    prefill_combine_body<D, T>(p, blockIdx.x, sh_scan);
+    prefill_combine_body<D, T, NSMAX>(p, blockIdx.x, sh_scan);
+}
+// The merge kernel for a launch whose partial buffers hold `slots` (slot, split) pairs.
+template <int D, class T>
+inline void launch_prefill_combine(const AttnParams& p, int slots, hipStream_t stream) {
+    const dim3 grid(prefill_combine_grid_of(p, slots)), block(256);
+    if (slots <= 2) hipLaunchKernelGGL((attn_prefill_combine<D, T, 2>), grid, block, 0, stream, p);
+    else if (slots <= 4) hipLaunchKernelGGL((attn_prefill_combine<D, T, 4>), grid, block, 0, stream, p);
+    else if (slots <= 8) hipLaunchKernelGGL((attn_prefill_combine<D, T, 8>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_prefill_combine<D, T, 16>), grid, block, 0, stream, p);
 }
 
-// Workgroups the merge kernel of a split prefill-shaped launch needs (0 = the launch never splits).
-inline int prefill_combine_grid(const AttnParams& p) {
-    const int slots = p.part_o ? p.split_slots : 1;
-    if (slots <= 1) return 0;
-    const int items = p.B < slots / 2 ? p.B : slots / 2;  // more active slots than this are never split
-    return items * p.H * ((p.Tq + PFC_ROWS - 1) / PFC_ROWS);
-}
 
 }  // namespace g4b

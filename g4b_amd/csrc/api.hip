@@ -262,6 +262,7 @@ static int fill_attn_params(const g4b_attn_args* a, g4b::AttnParams& p) {
     // a query wider than the cache type: f32 over f16 / bf16, f16 over bf16
     const bool q_wider = a->q_dtype == G4B_DT_F32 || (a->q_dtype == G4B_DT_F16 && a->kv_dtype == G4B_DT_BF16);
     p.q_split = (a->use_fp32_dot && q_wider) ? 1 : 0;
+    p.xcd_shift = 0;  // the decode kernels proper have one worker per workgroup, and workgroup i runs on XCD i % 8
     return G4B_OK;
 }
 
@@ -413,6 +414,7 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
         }
         if (m.nw) {
             pd.NW = m.nw;
+            pd.xcd_shift = -1;  // the workers of a mixed launch share their workgroups and the chip with the chunk: equal shares
             pd.part_o = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + pf_span);
             pd.part_ml = pd.part_o + decode_slots(a->B, a->G, m.nw) * (uint64_t)pd.R * pd.Tq * (uint64_t)a->D;
         }

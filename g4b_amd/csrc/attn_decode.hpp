@@ -29,13 +29,48 @@ constexpr int DEC_TILE = 32;  // keys per wave iteration
 
 G4B_DEV int slot_tiles(const SlotInfo& s) { return (s.window - s.klo + DEC_TILE - 1) / DEC_TILE; }
 G4B_DEV int slot_tiles(const AttnParams& p, int b) { return slot_tiles(slot_info(p, b)); }
-// floor(a * b / c) for a * b below 2^63; in 32 bits when the caller knows that a * b fits (`small`, the same in every
-// lane): a 64-bit division is some 150 instructions, and a decode worker makes two of them before its first load.
-G4B_DEV int64_t muldiv(int64_t a, int64_t b, int64_t c, bool small) {
-    if (small) return (int64_t)((uint32_t)a * (uint32_t)b / (uint32_t)c);
-    return a * b / c;
+// Share-out of the flat tile list over nw workers.  The odd XCDs of the chip stream from HBM more slowly than the even
+// ones (a decode batch with equal shares: workers on XCDs 0, 2, 4, 6 took 148 .. 160 us, those on 1, 3, 5, 7
+// 165 .. 172 us, on three boxes, and the slow half followed the hardware when the shares were swapped), and a launch
+// lasts as long as its slowest worker, so a worker on an even XCD gets 25 + XCD_SKEW parts of the list for every
+// 25 - XCD_SKEW on an odd one (batch of 64: 0.820 -> 0.835 of 8 TB/s; the odd XCDs still finish last, more slowly per
+// tile while the even ones take more of the memory system, so the gain is the shorter tail, not the 8 %).  Worker w
+// starts at tile floor(total * cum(w) / cum(nw)), cum(w) = 25 w + e(w) being the parts of the workers before it; unweighted (parity unknown, or fewer than two tiles per worker, where a share could come out empty)
+// cum(w) = w.
+constexpr int XCD_SKEW = 1;  // parts out of 25 taken from an odd XCD's worker and given to an even one's (2 measured the same, 3 worse)
+struct TileShares {
+    int64_t total;
+    int nw, shift;  // shift < 0: equal shares
+    bool small;     // total * cum(nw) fits 32 bits
+    G4B_DEV int64_t cum(int w) const {
+        if (shift < 0) return w;
+        const int period = 2 << shift, r = w & (period - 1);
+        return 25 * (int64_t)w + XCD_SKEW * (r <= period / 2 ? r : period - r);
+    }
+    G4B_DEV int64_t begin(int w) const {  // first tile of worker w; begin(nw) = total
+        const int64_t c = cum(w), cn = cum(nw);
+        if (small) return (int64_t)((uint32_t)total * (uint32_t)c / (uint32_t)cn);
+        return total * c / cn;
+    }
+    G4B_DEV int owner(int64_t x) const {  // the worker that owns tile x: the largest w with begin(w) <= x
+        const int64_t cn = cum(nw);
+        int64_t c;
+        if (small) c = (int64_t)(((uint32_t)(x + 1) * (uint32_t)cn - 1u) / (uint32_t)total);
+        else c = ((x + 1) * cn - 1) / total;
+        if (shift < 0) return (int)c;
+        int w = (int)(c / 25);
+        if (cum(w) > c) --w;
+        return w;
+    }
+};
+G4B_DEV TileShares tile_shares(const AttnParams& p, int total) {
+    TileShares s;
+    s.total = total;
+    s.nw = min(p.NW, total);  // never more workers than tiles: every worker below nw owns >= 1 tile
+    s.shift = (p.xcd_shift >= 0 && total >= 2 * s.nw) ? p.xcd_shift : -1;
+    s.small = (uint64_t)total * (uint64_t)(25 * (int64_t)s.nw + 4) < ((uint64_t)1 << 32);
+    return s;
 }
-
 template <int CL>
 G4B_DEV float pick(const f4& c, int e, int cls) {
     // element e*CL + cls of c without dynamic register indexing
@@ -314,11 +349,10 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
         total += G * tl;
     }
     total = wave_sum_i(total);
-    const int nw = min(p.NW, total);  // never more workers than tiles: every worker below nw owns >= 1 tile
-    if (w >= nw) return;
-    const bool small = (uint64_t)total * (uint64_t)nw < ((uint64_t)1 << 32);
-    const int64_t ws = muldiv(w, total, nw, small);
-    const int64_t we = muldiv(w + 1, total, nw, small);
+    const TileShares shares = tile_shares(p, total);
+    if (w >= shares.nw) return;
+    const int64_t ws = shares.begin(w);
+    const int64_t we = shares.begin(w + 1);
 
     int carry = 0;
     for (int b0 = 0; b0 < B; b0 += 64) {
@@ -457,18 +491,9 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
         return;
     }
     if (p.NW == 0) return;  // one wave owned the whole pair
-    const int nw = min(p.NW, total);
+    const TileShares shares = tile_shares(p, total);
     const int64_t fs = (int64_t)before + (int64_t)g * tl;
-    // worker that owns flat tile x: the largest w with floor(w * total / nw) <= x
-    const bool small = (uint64_t)total * (uint64_t)nw < ((uint64_t)1 << 32);  // (fs + tl) * nw <= total * nw
-    int w0, w1;
-    if (small) {
-        w0 = (int)(((uint32_t)(fs + 1) * (uint32_t)nw - 1u) / (uint32_t)total);
-        w1 = (int)(((uint32_t)(fs + tl) * (uint32_t)nw - 1u) / (uint32_t)total);
-    } else {
-        w0 = (int)(((fs + 1) * nw - 1) / total);
-        w1 = (int)(((fs + tl) * nw - 1) / total);
-    }
+    const int w0 = shares.owner(fs), w1 = shares.owner(fs + tl - 1);
     if (w0 == w1) return;  // a single worker owned the pair and wrote the output itself
 
     // partial of worker w for this pair and row: slot w + pair

@@ -354,6 +354,8 @@ struct AttnParams {
     int32_t kernel_mask;  // bit 0: main kernel, bit 1: merge kernel
     int32_t q_split;      // 1: a query wider than the cache type enters K Q^T as a hi + lo pair of operands
     int32_t pair_split;   // 1: a prefill launch that splits keys still pairs query tiles (prefill_map.hpp)
+    int32_t xcd_shift;    // decode workers: bit (worker >> xcd_shift) & 1 is the parity of the XCD the worker runs on;
+                          // < 0: unknown, every worker gets the same share of the tiles
     float c;     // softmax scale * log2(e)
 };
 

@@ -57,7 +57,20 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     const int half = p.D / 2;
     const int tpr = half / CPT;          // threads per token
     const int rows = 256 / tpr;          // tokens per workgroup
-    const int tt = blockIdx.x * rows + threadIdx.x / tpr;
+    // Workgroups go to the 8 XCDs round-robin by id, and the odd XCDs stream from HBM more slowly than the even ones
+    // (attn_decode.hpp): a launch of many token blocks deals 26 of every 50 to the even workgroups, so that both
+    // halves of the chip finish together; the odd workgroups left over leave at once.
+    int block = blockIdx.x;
+    if (p.even_blocks > 0) {
+        const int k = block >> 1;
+        if (block & 1) {
+            block = p.even_blocks + k;
+        } else {
+            if (k >= p.even_blocks) return;
+            block = k;
+        }
+    }
+    const int tt = block * rows + threadIdx.x / tpr;
     const int j0 = (threadIdx.x % tpr) * CPT;
     // threads beyond rows * tpr (tpr does not divide 256) would alias the next workgroup's first token
     if ((int)threadIdx.x >= rows * tpr || tt >= p.t) return;
@@ -160,9 +173,11 @@ hipError_t launch_rope(const RopeParams& p, hipStream_t stream) {
     const int jobs = p.H + 2 * p.G;
     int z = 1;
     while (z < 4 && z * 2 <= jobs && (int64_t)blocks * p.B * z < 256) z *= 2;
-    dim3 grid(blocks, p.B, z);
-    if (cpt == 4) G4B_LAUNCH_DOMINANT(rope_kernel<4>, grid, dim3(256), 0, stream, p);
-    else G4B_LAUNCH_DOMINANT(rope_kernel<8>, grid, dim3(256), 0, stream, p);
+    RopeParams pk = p;
+    pk.even_blocks = blocks >= 128 ? (blocks * 26 + 49) / 50 : 0;
+    dim3 grid(pk.even_blocks ? 2 * pk.even_blocks : blocks, p.B, z);
+    if (cpt == 4) G4B_LAUNCH_DOMINANT(rope_kernel<4>, grid, dim3(256), 0, stream, pk);
+    else G4B_LAUNCH_DOMINANT(rope_kernel<8>, grid, dim3(256), 0, stream, pk);
     return hipGetLastError();
 }
 

@@ -52,6 +52,10 @@ CASES = [
     # D / 16 does not divide the 256 threads of a workgroup: the spare threads must stay out of the next block's token
     ("chunk_d96", 2, 4, 2, 130, 96, [7, 3000]),
     ("chunk_d160", 1, 4, 1, 77, 160, [41]),
+    # 138 token blocks of 8 tokens, the last one ragged: enough blocks for the launch to deal them unevenly to the
+    # workgroups of even and odd XCDs
+    ("prompt_d256", 1, 8, 2, 1100, 256, [3]),
+    ("prompt_two_slots_d128", 2, 4, 2, 2100, 128, [0, 50000]),
 ]
 
 
@@ -82,16 +86,18 @@ def test_apply_rope_on_16_bit_scratchpads(rope, dtype, tol):
 
 @pytest.mark.parametrize("Dv", [256, 128, 512])
 @pytest.mark.parametrize("cache_dtype", [torch.float16, torch.bfloat16])
-def test_fused_append_equals_rope_then_two_appends(rope, Dv, cache_dtype):
-    """One launch == apply_rope + add_kv_to_cache(k) + add_kv_to_cache(v, v_rsos) with phase skip and ring wrap."""
+@pytest.mark.parametrize("t,T", [(40, 97), (1030, 1200)], ids=["chunk", "prompt"])
+def test_fused_append_equals_rope_then_two_appends(rope, Dv, cache_dtype, t, T):
+    """One launch == apply_rope + add_kv_to_cache(k) + add_kv_to_cache(v, v_rsos) with phase skip and ring wrap (the
+    prompt-sized case has enough token blocks for the uneven deal between even and odd XCDs)."""
     from g4b_amd.kernels.add_kv_to_cache import add_kv_to_cache
 
-    B, H, G, t, D, T = 4, 8, 2, 40, 256, 97
+    B, H, G, D = 4, 8, 2, 256
     q, k, freqs, q_rsos, k_rsos, qw, kw = _case(B, H, G, t, D, seed=23, engine_layout=True)
     gen = torch.Generator().manual_seed(24)
     v = torch.randn(B, t, G, Dv, generator=gen).cuda().permute(0, 2, 1, 3)
     v_rsos = (v ** 2).sum(-1)
-    offs = i32([0, 80, 97 * 5 + 90, 3])
+    offs = i32([0, 80, T * 5 + T - 7, 3])
     phase = u8([1, 1, 1, 2])
     kc0 = torch.randn(B, G, T, D, generator=gen).to(cache_dtype).cuda()
     vc0 = torch.randn(B, G, T, Dv, generator=gen).to(cache_dtype).cuda()

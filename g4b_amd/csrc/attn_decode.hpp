@@ -48,17 +48,22 @@ struct TileShares {
         return 25 * (int64_t)w + XCD_SKEW * (r <= period / 2 ? r : period - r);
     }
     G4B_DEV int64_t begin(int w) const {  // first tile of worker w; begin(nw) = total
-        const int64_t c = cum(w), cn = cum(nw);
-        if (small) return (int64_t)((uint32_t)total * (uint32_t)c / (uint32_t)cn);
-        return total * c / cn;
+        if (small) {  // the common case in 32-bit arithmetic throughout
+            const uint32_t c = shift < 0 ? (uint32_t)w : (uint32_t)cum(w), cn = shift < 0 ? (uint32_t)nw : (uint32_t)cum(nw);
+            return (int64_t)((uint32_t)total * c / cn);
+        }
+        return total * cum(w) / cum(nw);
     }
     G4B_DEV int owner(int64_t x) const {  // the worker that owns tile x: the largest w with begin(w) <= x
-        const int64_t cn = cum(nw);
         int64_t c;
-        if (small) c = (int64_t)(((uint32_t)(x + 1) * (uint32_t)cn - 1u) / (uint32_t)total);
-        else c = ((x + 1) * cn - 1) / total;
+        if (small) {
+            const uint32_t cn = shift < 0 ? (uint32_t)nw : (uint32_t)cum(nw);
+            c = (int64_t)(((uint32_t)(x + 1) * cn - 1u) / (uint32_t)total);
+        } else {
+            c = ((x + 1) * cum(nw) - 1) / total;
+        }
         if (shift < 0) return (int)c;
-        int w = (int)(c / 25);
+        int w = (int)((uint32_t)c / 25u);  // c < 25 nw + 4
         if (cum(w) > c) --w;
         return w;
     }

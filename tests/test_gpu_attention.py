@@ -61,8 +61,10 @@ def test_decode_matches_oracle_split_and_unsplit(fa, case, scale):
     assert bool((diff <= 5e-4 + 2e-3 * o.float().abs()).all()), diff.max().item()
 
 
-@pytest.mark.parametrize("num_workers", [1, 3, 64, 777, 4096])
+@pytest.mark.parametrize("num_workers", [1, 3, 64, 100, 153, 154, 777, 4096])
 def test_decode_any_worker_count_gives_the_same_answer(fa, num_workers):
+    """306 tiles in all: up to 153 workers the shares are weighted by the parity of the worker's XCD (at least two tiles
+    per worker), from 154 on they are equal, from 306 on every worker has one tile."""
     B, H, G, D, W = 5, 8, 2, 256, 2048
     q, k, v, o = make_case(B, H, G, 1, D, W, seed=2)
     tds = [1, 33, 700, 2048, 2048 + 300]

@@ -39,31 +39,25 @@ G4B_DEV int slot_tiles(const AttnParams& p, int b) { return slot_tiles(slot_info
 // cum(w) = w.
 constexpr int XCD_SKEW = 1;  // parts out of 25 taken from an odd XCD's worker and given to an even one's (2 measured the same, 3 worse)
 struct TileShares {
-    int64_t total;
-    int nw, shift;  // shift < 0: equal shares
-    bool small;     // total * cum(nw) fits 32 bits
-    G4B_DEV int64_t cum(int w) const {
-        if (shift < 0) return w;
+    int total, nw, shift;  // shift < 0: equal shares
+    uint32_t cn;           // cum(nw)
+    bool small;            // total * cum(nw) fits 32 bits
+    G4B_DEV uint32_t cum(int w) const {
+        if (shift < 0) return (uint32_t)w;
         const int period = 2 << shift, r = w & (period - 1);
-        return 25 * (int64_t)w + XCD_SKEW * (r <= period / 2 ? r : period - r);
+        return 25u * (uint32_t)w + (uint32_t)(XCD_SKEW * (r <= period / 2 ? r : period - r));
     }
     G4B_DEV int64_t begin(int w) const {  // first tile of worker w; begin(nw) = total
-        if (small) {  // the common case in 32-bit arithmetic throughout
-            const uint32_t c = shift < 0 ? (uint32_t)w : (uint32_t)cum(w), cn = shift < 0 ? (uint32_t)nw : (uint32_t)cum(nw);
-            return (int64_t)((uint32_t)total * c / cn);
-        }
-        return total * cum(w) / cum(nw);
+        const uint32_t c = cum(w);
+        if (small) return (int64_t)((uint32_t)total * c / cn);  // the common case in 32-bit arithmetic throughout
+        return (int64_t)((uint64_t)total * c / cn);
     }
     G4B_DEV int owner(int64_t x) const {  // the worker that owns tile x: the largest w with begin(w) <= x
-        int64_t c;
-        if (small) {
-            const uint32_t cn = shift < 0 ? (uint32_t)nw : (uint32_t)cum(nw);
-            c = (int64_t)(((uint32_t)(x + 1) * cn - 1u) / (uint32_t)total);
-        } else {
-            c = ((x + 1) * cum(nw) - 1) / total;
-        }
+        uint32_t c;
+        if (small) c = ((uint32_t)(x + 1) * cn - 1u) / (uint32_t)total;
+        else c = (uint32_t)(((uint64_t)(x + 1) * cn - 1u) / (uint32_t)total);
         if (shift < 0) return (int)c;
-        int w = (int)((uint32_t)c / 25u);  // c < 25 nw + 4
+        int w = (int)(c / 25u);  // c < 25 nw + 4
         if (cum(w) > c) --w;
         return w;
     }
@@ -73,7 +67,8 @@ G4B_DEV TileShares tile_shares(const AttnParams& p, int total) {
     s.total = total;
     s.nw = min(p.NW, total);  // never more workers than tiles: every worker below nw owns >= 1 tile
     s.shift = (p.xcd_shift >= 0 && total >= 2 * s.nw) ? p.xcd_shift : -1;
-    s.small = (uint64_t)total * (uint64_t)(25 * (int64_t)s.nw + 4) < ((uint64_t)1 << 32);
+    s.cn = s.cum(s.nw);
+    s.small = (uint64_t)(uint32_t)total * s.cn < ((uint64_t)1 << 32);
     return s;
 }
 template <int CL>

@@ -94,16 +94,17 @@ uint64_t decode_slots(int B, int G, int nw) { return (uint64_t)nw + (uint64_t)B 
 constexpr int kPrefillFillWorkgroups = 256;
 constexpr int kPrefillMaxSplitSlots = 64;
 int prefill_rows_per_workgroup(int /*D*/) { return 128; }
-// A slot that brings at least half as many query tiles as the chip has compute units is not split tile by tile; the
-// 128 / 256 kernel then still has only a quarter to a half of the units busy with its pairs of query tiles, and cuts
-// the key tiles of every pair into two or three equal spans instead (measured, one slot, causal from an empty cache:
-// S = 3072 95 -> 64 us, S = 4096 119 -> 89 us; for shorter prompts, which the tile-by-tile split already serves, it
-// measured worse: S = 1024 25 -> 32 us).  The 512 kernel gives every workgroup one query tile.
+// A slot that brings at least a third as many query tiles as the chip has compute units is not split tile by tile
+// (under the causal mask equal splits of every tile leave the launch as long as half of its heaviest tile); the
+// 128 / 256 kernel pairs its query tiles instead and cuts the key tiles of every pair into two to five spans of equal
+// cost (measured, one slot, causal from an empty cache: S = 1408 31.5 -> 25.2 us, S = 2048 38.9 -> 33.9 us,
+// S = 3072 95 -> 55 us, S = 4096 119 -> 78 us; shorter prompts measured worse that way, S = 1280 32.0 -> 33.6 us wall
+// and S = 1024 30.2 -> 33.4 us, for the wider merge).  The 512 kernel gives every workgroup one query tile.
 bool prefill_pair_split(int H, int G, int Tq, int D) {
     const int R = H / G, bm = prefill_rows_per_workgroup(D);
     if (D == 512 || R < 1 || bm % R) return false;
     const int tokb = bm / R, nq = (Tq + tokb - 1) / tokb;
-    return (int64_t)nq * G * 2 > kPrefillFillWorkgroups && (int64_t)((nq + 1) / 2) * G * 2 <= kPrefillFillWorkgroups;
+    return (int64_t)nq * G * 3 >= kPrefillFillWorkgroups && (int64_t)((nq + 1) / 2) * G * 2 <= kPrefillFillWorkgroups;
 }
 // One (slot, key split) pair of a prefill-shaped launch: its rows in the cache's 16-bit type, normalised by the split's
 // own sum, then (reference, sum) per row in fp32.

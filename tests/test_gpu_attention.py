@@ -471,14 +471,16 @@ def test_argument_errors_follow_the_reference(fa):
 
 
 @pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("Tq", [1000, 400])
 @pytest.mark.parametrize("case", ["from_scratch", "on_context", "two_active", "per_query_window", "full_stage", "bf16"])
-def test_prefill_pairs_of_query_tiles_cut_into_key_spans(fa, D, case):
-    """A slot that brings between a quarter and a half of the chip's compute units in pairs of query tiles: the key tiles
-    of every pair (heavy tile, then light tile) are cut into two or three equal spans, one workgroup each; a tile that
-    lies wholly in one span is written straight to o, the others are merged.  H/G = 16 makes a query tile 8 tokens, so
-    1000 tokens are 125 tiles = 63 pairs per kv head."""
-    print(f"pair split {case} D={D}", flush=True)
-    H, G, Tq, kv_ctx = 32, 2, 1000, 1300
+def test_prefill_pairs_of_query_tiles_cut_into_key_spans(fa, D, case, Tq):
+    """A slot that brings between a third of the chip's compute units and all of them in query tiles: the tiles are
+    paired and the key tiles of every pair (heavy tile, then light tile) are cut into two to five spans of equal cost,
+    one workgroup each; a tile that lies wholly in one span is written straight to o, the others are merged.  H/G = 16
+    makes a query tile 8 tokens, so 1000 tokens are 125 tiles = 63 pairs per kv head (two spans each) and 400 tokens 50
+    tiles = 25 pairs (five spans each)."""
+    print(f"pair split {case} D={D} Tq={Tq}", flush=True)
+    H, G, kv_ctx = 32, 2, 1300
     B = 3 if case == "two_active" else 2
     dtype = torch.bfloat16 if case == "bf16" else torch.float16
     q, k, v, o = make_case(B, H, G, Tq, D, kv_ctx, seed=len(case) + D, dtype=dtype)

@@ -83,7 +83,10 @@ def test_workspace_size_formula(native):
     # than 256 workgroups (16 query tiles x 2 kv heads here -> 8 pairs), nothing when the shape fills the chip by itself
     assert lib.g4b_attn_workspace_bytes(1, 8, 2, 512, 256, 0) == 8 * 8 * 512 * (256 * 2 + 8)
     assert lib.g4b_attn_workspace_bytes(33, 8, 2, 512, 256, 0) == 8 * 8 * 512 * (256 * 2 + 8)  # independent of B
-    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 2048, 256, 0) == 2 * 8 * 2048 * (256 * 2 + 8)
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 1024, 256, 0) == 4 * 8 * 1024 * (256 * 2 + 8)  # 32 tiles x 2 kv heads -> 4 pairs
+    # from a third of the chip's units in query tiles on, the tiles are paired and the pairs cut into spans:
+    # 2048 tokens are 32 pairs x 2 kv heads -> 4 spans each
+    assert lib.g4b_attn_workspace_bytes(1, 8, 2, 2048, 256, 0) == 4 * 8 * 2048 * (256 * 2 + 8)
     assert lib.g4b_attn_workspace_bytes(1, 8, 2, 8192, 256, 0) == 0
 
 

@@ -2,8 +2,9 @@
 // (R = H/G heads x Tq tokens), the KV cache is streamed from HBM exactly once per pair.
 //
 // Work decomposition.  Every in-phase slot contributes ceil(keys / 32) tiles per kv head; the
-// tiles of all pairs form one flat list that is dealt evenly to NW single-wave workgroups
-// (worker w owns flat tiles [w*T/NW, (w+1)*T/NW)).  The split is computed on the device from
+// tiles of all pairs form one flat list that is dealt to NW single-wave workgroups in contiguous
+// runs (worker w owns flat tiles [begin(w), begin(w+1)), TileShares below: equal shares, or 26 : 24
+// between workers on even and odd XCDs).  The split is computed on the device from
 // time_dim_sizes, so the grid is static while the balance follows the real lengths.  A worker
 // whose range covers a whole pair writes the output directly; otherwise it leaves an
 // un-normalised fp32 partial (acc, running max, running sum) in workspace slot (w + pair) and a
@@ -35,8 +36,8 @@ G4B_DEV int slot_tiles(const AttnParams& p, int b) { return slot_tiles(slot_info
 // lasts as long as its slowest worker, so a worker on an even XCD gets 25 + XCD_SKEW parts of the list for every
 // 25 - XCD_SKEW on an odd one (batch of 64: 0.820 -> 0.835 of 8 TB/s; the odd XCDs still finish last, more slowly per
 // tile while the even ones take more of the memory system, so the gain is the shorter tail, not the 8 %).  Worker w
-// starts at tile floor(total * cum(w) / cum(nw)), cum(w) = 25 w + e(w) being the parts of the workers before it; unweighted (parity unknown, or fewer than two tiles per worker, where a share could come out empty)
-// cum(w) = w.
+// starts at tile floor(total * cum(w) / cum(nw)), cum(w) = 25 w + e(w) being the parts of the workers before it;
+// unweighted (parity unknown, or fewer than two tiles per worker, where a share could come out empty) cum(w) = w.
 constexpr int XCD_SKEW = 1;  // parts out of 25 taken from an odd XCD's worker and given to an even one's (2 measured the same, 3 worse)
 struct TileShares {
     int total, nw, shift;  // shift < 0: equal shares

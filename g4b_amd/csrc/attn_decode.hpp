@@ -43,17 +43,17 @@ struct TileShares {
     int total, nw, shift;  // shift < 0: equal shares
     uint32_t cn;           // cum(nw)
     bool small;            // total * cum(nw) fits 32 bits
-    G4B_DEV uint32_t cum(int w) const {
+    __host__ __device__ uint32_t cum(int w) const {
         if (shift < 0) return (uint32_t)w;
         const int period = 2 << shift, r = w & (period - 1);
         return 25u * (uint32_t)w + (uint32_t)(XCD_SKEW * (r <= period / 2 ? r : period - r));
     }
-    G4B_DEV int64_t begin(int w) const {  // first tile of worker w; begin(nw) = total
+    __host__ __device__ int64_t begin(int w) const {  // first tile of worker w; begin(nw) = total
         const uint32_t c = cum(w);
         if (small) return (int64_t)((uint32_t)total * c / cn);  // the common case in 32-bit arithmetic throughout
         return (int64_t)((uint64_t)total * c / cn);
     }
-    G4B_DEV int owner(int64_t x) const {  // the worker that owns tile x: the largest w with begin(w) <= x
+    __host__ __device__ int owner(int64_t x) const {  // the worker that owns tile x: the largest w with begin(w) <= x
         uint32_t c;
         if (small) c = ((uint32_t)(x + 1) * cn - 1u) / (uint32_t)total;
         else c = (uint32_t)(((uint64_t)(x + 1) * cn - 1u) / (uint32_t)total);
@@ -63,15 +63,18 @@ struct TileShares {
         return w;
     }
 };
-G4B_DEV TileShares tile_shares(const AttnParams& p, int total) {
+// num_workers: the launch's worker count; xcd_shift: AttnParams::xcd_shift.  (Host-callable so that the arithmetic the
+// workers and the merge kernel share can be brute-forced on the CPU.)
+__host__ __device__ inline TileShares make_tile_shares(int num_workers, int xcd_shift, int total) {
     TileShares s;
     s.total = total;
-    s.nw = min(p.NW, total);  // never more workers than tiles: every worker below nw owns >= 1 tile
-    s.shift = (p.xcd_shift >= 0 && total >= 2 * s.nw) ? p.xcd_shift : -1;
+    s.nw = num_workers < total ? num_workers : total;  // never more workers than tiles: every worker below nw owns >= 1 tile
+    s.shift = (xcd_shift >= 0 && total >= 2 * s.nw) ? xcd_shift : -1;
     s.cn = s.cum(s.nw);
     s.small = (uint64_t)(uint32_t)total * s.cn < ((uint64_t)1 << 32);
     return s;
 }
+G4B_DEV TileShares tile_shares(const AttnParams& p, int total) { return make_tile_shares(p.NW, p.xcd_shift, total); }
 template <int CL>
 G4B_DEV float pick(const f4& c, int e, int cls) {
     // element e*CL + cls of c without dynamic register indexing

@@ -107,6 +107,16 @@ def traffic_from_counters(prof_dir: str) -> dict:
 H, G, D = 8, 2, 256
 SCALE = 1.0 / 16.0
 
+# Where split partials go: "caller" = a workspace tensor sized with workspace_bytes() next to the engine's own partial
+# buffers (what the integration notes recommend), "static" = the library's own scratch array (what the wrappers take
+# when no workspace is passed: same kernels, a few microseconds slower per split launch on this board).
+WORKSPACE_MODE = "caller"
+
+
+def WORKSPACE_OF(ws):
+    return "static" if WORKSPACE_MODE == "static" or ws is None else ws
+
+
 
 def host_cpu_model() -> str:
     try:
@@ -186,7 +196,7 @@ class BatchedDecode(Workload):
         if plan is None:
             plan = self.plans[kernel_mask] = self.fa2.plan_flash_attention(
                 self.q, self.k, self.v, self.o, self.tds, self.phase, self.kv_ctx, self.fa2.PHASE_DECODE,
-                scale=SCALE, window_sizes=self.win, workspace=self.ws, kernel_mask=kernel_mask,
+                scale=SCALE, window_sizes=self.win, workspace=WORKSPACE_OF(self.ws), kernel_mask=kernel_mask,
             )
         plan.launch()
 
@@ -233,7 +243,7 @@ class SingleDecode(Workload):
         self.plans = {
             (c, km): fa2.plan_flash_attention(
                 self.q[c : c + 1], self.k[c : c + 1], self.v[c : c + 1], self.o[c : c + 1], self.tds, self.phase,
-                n, fa2.PHASE_DECODE, scale=SCALE, workspace=self.ws, kernel_mask=km,
+                n, fa2.PHASE_DECODE, scale=SCALE, workspace=WORKSPACE_OF(self.ws), kernel_mask=km,
             )
             for c in range(copies) for km in (0, 1)
         }
@@ -310,6 +320,8 @@ class Prefill(Workload):
             pairs = w * (w + 1) // 2 + (S - w) * w
         self.pairs = pairs
         self.plan = None
+        need = fa2.workspace_bytes(1, H, G, S, D_)
+        self.ws = torch.empty(need, dtype=torch.uint8, device=device) if need and WORKSPACE_MODE == "caller" else None
         self.flops = 4 * H * D_ * pairs
         self.bytes = (2 * H * S * D_ + 2 * G * S * D_) * 2
         self.units = self.flops
@@ -318,7 +330,7 @@ class Prefill(Workload):
         if self.plan is None:
             self.plan = self.fa2.plan_flash_attention(
                 self.q, self.k, self.v, self.o, self.tds, self.phase, self.S, self.fa2.PHASE_PREFILL,
-                scale=SCALE, query_window=self.qw,
+                scale=SCALE, query_window=self.qw, workspace=WORKSPACE_OF(self.ws),
             )
         self.plan.launch()
 
@@ -669,6 +681,9 @@ def main():
                     help="untimed steps first; the board needs some 20 ms of load before its clocks settle")
     ap.add_argument("--workload", default="decode_batched", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extra", action="store_true", help="time the primary workload only")
+    ap.add_argument("--workspace", choices=("static", "caller"), default="caller",
+                    help="split partials in a caller-owned workspace tensor (default) or in the library's static scratch "
+                         "(what the wrappers take when no workspace is passed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-from", metavar="DIR",
                     help="no GPU work: read DIR/pmc_FETCH_SIZE_<workload> and DIR/pmc_WRITE_SIZE_<workload> (rocprofv3 "
@@ -683,6 +698,8 @@ def main():
     if args.traffic_from:
         print(json.dumps(traffic_from_counters(args.traffic_from), indent=1, sort_keys=True))
         return
+    global WORKSPACE_MODE
+    WORKSPACE_MODE = args.workspace
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the attention path shards by slot or kv head with "
                  "no exchange; nothing here uses a second device). Run with --gpus 1.")

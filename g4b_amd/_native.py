@@ -12,9 +12,10 @@ G4B_ERR_INVALID_ARGUMENT = -1
 G4B_ERR_UNSUPPORTED = -2
 G4B_ERR_WORKSPACE = -3
 G4B_ERR_LAUNCH = -4
+G4B_ERR_BUSY = -5
 
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class AttnArgs(C.Structure):
@@ -189,11 +190,17 @@ def last_error() -> str:
     return load().g4b_last_error().decode()
 
 
+class ScratchBusyError(ValueError):
+    """g4b_attn_forward_static_scratch found the static scratch in use by unfinished work on another stream."""
+
+
 def check(status: int) -> None:
     """Map a g4b_status to the exception the reference raises for the same mistake."""
     if status == G4B_OK:
         return
     msg = last_error()
+    if status == G4B_ERR_BUSY:
+        raise ScratchBusyError(msg)
     if status in (G4B_ERR_INVALID_ARGUMENT, G4B_ERR_WORKSPACE):
         raise ValueError(msg)
     if status == G4B_ERR_UNSUPPORTED:

@@ -26,6 +26,13 @@ thread_local char g_err[512] = "";
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void* g_scratch_ptr[kMaxDevices] = {};
+// The stream whose launches last used the array on each device.  A launch on another stream may only follow when
+// everything enqueued on that stream has finished (two launches in flight would write their partials over each other's).
+struct ScratchOwner {
+    hipStream_t stream = nullptr;
+    bool valid = false;
+};
+ScratchOwner g_scratch_owner[kMaxDevices];
 
 // Device address of `scratch` on the current device, looked up once per device.
 hipError_t static_scratch_ptr(void** out) {
@@ -43,6 +50,27 @@ hipError_t static_scratch_ptr(void** out) {
     }
     *out = g_scratch_ptr[dev];
     return hipSuccess;
+}
+
+// Claim the array of the current device for a launch on `stream`: true when the launch may use it.  A launch that is
+// being recorded into a graph is let through untracked (when it will run is not known here; whoever replays the graph
+// keeps it apart from other launches that use the array).
+bool claim_static_scratch(hipStream_t stream) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return true;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ScratchOwner& o = g_scratch_owner[dev];
+    if (o.valid && o.stream == stream) return true;  // the common case costs no runtime call
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) == hipSuccess && cs == hipStreamCaptureStatusActive) return true;
+    if (o.valid) {
+        const hipError_t e = hipStreamQuery(o.stream);
+        if (e == hipErrorNotReady) return false;
+        if (e != hipSuccess) (void)hipGetLastError();  // the stream is gone: nothing of it is pending
+    }
+    o.stream = stream;
+    o.valid = true;
+    return true;
 }
 
 // g4b_profile_begin .. g4b_profile_end: one (start, stop) event pair per timed call of this thread
@@ -228,6 +256,9 @@ static int fill_attn_params(const g4b_attn_args* a, g4b::AttnParams& p) {
     if ((int64_t)a->KV_CTX * a->D * (a->kv_dtype == G4B_DT_F32 ? 4 : 2) >= (int64_t)1 << 31)
         return fail(G4B_ERR_UNSUPPORTED, "one (slot, kv head) of the cache must stay below 2 GiB");
     if (a->num_workers < 0 || a->num_workers > (1 << 20)) return fail(G4B_ERR_INVALID_ARGUMENT, "num_workers out of range");
+    // the streaming kernels count the 32-key tiles of all (slot, kv head) pairs in 32 bits
+    if ((int64_t)a->B * a->G * (((int64_t)a->KV_CTX + 31) / 32) >= (int64_t)1 << 31)
+        return fail(G4B_ERR_UNSUPPORTED, "B * G * ceil(KV_CTX / 32) must stay below 2^31");
 
     p = g4b::AttnParams{};
     p.q = a->q;
@@ -457,6 +488,9 @@ int g4b_attn_forward_static_scratch(const g4b_attn_args* a, void* stream) {
         void* ptr = nullptr;
         const hipError_t e = static_scratch_ptr(&ptr);
         if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "static scratch: %s", hipGetErrorString(e));
+        if (!claim_static_scratch(static_cast<hipStream_t>(stream)))
+            return fail(G4B_ERR_BUSY, "the static scratch of this GPU is in use by work on another stream that has not finished; "
+                        "order the streams, or give this call a workspace of its own (g4b_attn_forward)");
         b.workspace = ptr;
         b.workspace_bytes = kStaticScratchBytes;
     }

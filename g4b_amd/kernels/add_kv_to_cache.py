@@ -72,5 +72,5 @@ def add_kv_to_cache(
     a.phase = phase
     a.rmsnorm_eps = float(rmsnorm_eps)
     lib = _native.load()
-    _native.check(lib.g4b_kv_append(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    _native.check(lib.g4b_kv_append(C.byref(a), C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream))))
     return None

@@ -48,6 +48,6 @@ def advance_decode_state(input_token_ids, out_token_ids, cache_offsets, time_dim
     a.B = B
     lib = _native.load()
     _native.check(
-        lib.g4b_advance_decode_state(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream)))
+        lib.g4b_advance_decode_state(C.byref(a), C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream)))
     )
     return None

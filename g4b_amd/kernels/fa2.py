@@ -9,6 +9,7 @@ Same public surface as the reference module: the ``STAGE_*`` / ``PHASE_*`` const
 from __future__ import annotations
 
 import ctypes as C
+import warnings
 
 from .. import _native
 from . import utils as U
@@ -26,6 +27,27 @@ PHASE_PREFILL = 1
 PHASE_DECODE = 2
 
 MAX_DECODE_ROWS = 16  # (H/G) * Tq up to which a launch takes the split-KV streaming kernel
+
+_warned = set()
+
+
+def _warn_once(key: str, message: str) -> None:
+    if key not in _warned:
+        _warned.add(key)
+        warnings.warn(message, RuntimeWarning, stacklevel=3)
+
+
+def _launch(entry, args_ref, stream, implicit_static: bool) -> None:
+    """The C call.  A call that took the library's static scratch by default (``workspace=None``) and finds it in use
+    by unfinished work on another stream runs without scratch instead (no key split: correct, slower) and says so
+    once; a call that asked for it (``workspace="static"``) gets the error."""
+    rc = entry(args_ref, stream)
+    if rc == _native.G4B_ERR_BUSY and implicit_static:
+        _warn_once("busy", "flash_attention: the library's static scratch is in use on another stream; this launch runs "
+                   "without a key split.  Pass workspace= (see workspace_bytes) to calls that overlap on one GPU.")
+        rc = _native.load().g4b_attn_forward(args_ref, stream)
+    if rc:
+        _native.check(rc)
 
 
 def workspace_bytes(B: int, H: int, G: int, Tq: int, D: int, num_workers: int = 0) -> int:
@@ -172,13 +194,17 @@ def _bind(
     elif workspace is None or isinstance(workspace, str):
         # Nothing is ever allocated here: the split partials go to the library's own scratch array
         # (g4b_attn_forward_static_scratch).  A decode-shaped launch splits only when the reference's split buffers
-        # were passed (fa2.py:658); a prefill shape whose in-phase slots may bring fewer workgroups than the chip has
+        # were passed (fa2.py:658) or the array was asked for by name; a prefill shape whose in-phase slots may bring fewer workgroups than the chip has
         # compute units (chunked prefill, short prompts) splits every item's keys.  A launch whose partials would not
         # fit the array runs unsplit.
         decode_shaped = (H // G) * Tq <= MAX_DECODE_ROWS
         need = workspace_bytes(B, H, G, Tq, D, num_workers if decode_shaped else 0)
-        wanted = need > 0 and (max_kv_splits > 1 if decode_shaped else True)
+        wanted = need > 0 and (workspace == "static" or not decode_shaped or max_kv_splits > 1)
         static = wanted and need <= int(lib.g4b_static_scratch_bytes())
+        if wanted and not static:
+            _warn_once("too big", f"flash_attention: this launch would split keys through {need} bytes of partials, more than "
+                       f"the library's static scratch holds ({int(lib.g4b_static_scratch_bytes())}); it runs without a key "
+                       "split.  Pass workspace= (see workspace_bytes) to split it.")
     else:
         ws = workspace
     if ws is not None:
@@ -278,7 +304,7 @@ def flash_attention(
         workspace=workspace, num_workers=num_workers, kernel_mask=kernel_mask, on_band_block=on_band_block,
         decode_q=decode_q, decode_o=decode_o, decode_phase=decode_phase,
     )
-    _native.check(entry(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    _launch(entry, C.byref(a), C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream)), workspace is None)
     return None, None
 
 
@@ -303,18 +329,20 @@ class AttentionPlan:
     plan holds references to the tensors it points into.
     """
 
-    def __init__(self, args, keep, entry):
+    def __init__(self, args, keep, entry, implicit_static=False):
         self._args, self._keep, self._entry = args, keep, entry
+        self._implicit_static = implicit_static
         self._ref = C.byref(args)
 
     def launch(self, stream=None) -> None:
-        rc = self._entry(self._ref, C.c_void_p(U.current_stream() if stream is None else int(stream)))
+        st = C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream))
+        rc = self._entry(self._ref, st)
         if rc:
-            _native.check(rc)
+            _launch(self._entry, self._ref, st, self._implicit_static)  # the slow path: fall back or raise
 
 
 def plan_flash_attention(*args, **kwargs) -> AttentionPlan:
     """Same arguments as :func:`flash_attention`, positional or by keyword (``stream`` is ignored: it is given to
     ``launch``); returns an :class:`AttentionPlan`."""
     kwargs.pop("stream", None)
-    return AttentionPlan(*_bind_call(*args, **kwargs))
+    return AttentionPlan(*_bind_call(*args, **kwargs), implicit_static=kwargs.get("workspace") is None)

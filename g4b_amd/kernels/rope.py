@@ -68,7 +68,7 @@ def apply_rope(q, k, rope_freqs, time_dim_offsets, q_rsos, k_rsos, q_rmsnorm_w, 
     """
     a, _ = _bind(q, k, rope_freqs, time_dim_offsets, q_rsos, k_rsos, q_rmsnorm_w, k_rmsnorm_w, rmsnorm_eps)
     lib = _native.load()
-    _native.check(lib.g4b_rope(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    _native.check(lib.g4b_rope(C.byref(a), C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream))))
     return None
 
 
@@ -119,7 +119,7 @@ def apply_rope_and_append(
         a.user_phase_stride = U.strides_of(user_phase)[0]
     a.Dv, a.T, a.phase, a.k_writeback = Dv, T, phase, 1 if k_writeback else 0
     lib = _native.load()
-    _native.check(lib.g4b_rope(C.byref(a), C.c_void_p(U.current_stream() if stream is None else int(stream))))
+    _native.check(lib.g4b_rope(C.byref(a), C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream))))
     return None
 
 
@@ -137,7 +137,7 @@ def populate_rope_frequencies(out, freq_scalars, freq_base: float, *, stream=Non
     _native.check(
         lib.g4b_rope_frequencies(
             C.c_void_p(out.data_ptr()), C.c_void_p(sc_ptr), n, U.strides_of(out)[0], sc_stride, float(freq_base),
-            C.c_void_p(U.current_stream() if stream is None else int(stream)),
+            C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream)),
         )
     )
     return None

@@ -81,9 +81,15 @@ def set_stream(stream) -> None:
     _stream_override = stream
 
 
+def stream_handle(stream) -> int:
+    """hipStream_t of a ``stream=`` argument: an int, a ``torch.cuda.Stream`` (``cuda_stream``) or a g4b stream
+    (``handle``, ``g4b/device.py:99``)."""
+    return int(getattr(stream, "cuda_stream", getattr(stream, "handle", stream)))
+
+
 def current_stream() -> int:
     if _stream_override is not None:
-        return int(getattr(_stream_override, "cuda_stream", getattr(_stream_override, "handle", _stream_override)))
+        return stream_handle(_stream_override)
     try:
         import torch
 

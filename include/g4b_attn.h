@@ -24,14 +24,15 @@
 extern "C" {
 #endif
 
-#define G4B_ATTN_ABI_VERSION 3
+#define G4B_ATTN_ABI_VERSION 4
 
 enum g4b_status {
     G4B_OK = 0,
     G4B_ERR_INVALID_ARGUMENT = -1, /* shape / stride / dtype / value check failed (reference: tl.static_assert) */
     G4B_ERR_UNSUPPORTED = -2,      /* valid in the reference, not built here (e.g. head_dim above 1024, a mixed launch at head_dim 128) */
     G4B_ERR_WORKSPACE = -3,        /* workspace missing or too small for the requested split-KV launch */
-    G4B_ERR_LAUNCH = -4            /* the HIP runtime refused the launch (no device, bad stream, ...) */
+    G4B_ERR_LAUNCH = -4,           /* the HIP runtime refused the launch (no device, bad stream, ...) */
+    G4B_ERR_BUSY = -5              /* g4b_attn_forward_static_scratch: the array is in use by unfinished work on another stream */
 };
 
 enum g4b_dtype { G4B_DT_F16 = 0, G4B_DT_BF16 = 1, G4B_DT_F32 = 2 };
@@ -170,7 +171,10 @@ uint64_t g4b_attn_mixed_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t
  * than that is refused with G4B_ERR_WORKSPACE (the limit covers every prefill shape up to head dimension 512 and
  * decode batches of about a thousand (slot, kv head) pairs at the default worker count).  No kernel reads scratch
  * that the same call has not written, so nothing is cleared between calls; all calls on one GPU share the array, so
- * calls that overlap on one GPU (two streams, two threads) race -- serialise them or give one of them a workspace.
+ * calls that overlap on one GPU would race.  The library remembers, per GPU, the stream of the last call that used the
+ * array: a call on another stream while that stream still has unfinished work is refused with G4B_ERR_BUSY (wait for
+ * the first stream, or give one of the calls a workspace through g4b_attn_forward).  Calls recorded into a graph are
+ * not tracked -- whoever replays graphs concurrently keeps their launches apart.
  *
  * g4b_static_scratch_init looks the array's device address up for the current device (the first
  * g4b_attn_forward_static_scratch on a device does the same); call it once per device at load when the first launch

@@ -286,3 +286,24 @@ def test_static_scratch_entry_point_checks_its_arguments(native):
     a.workspace = 4096
     assert lib.g4b_attn_forward_static_scratch(ctypes.byref(a), None) == native.G4B_ERR_INVALID_ARGUMENT
     assert "workspace must be NULL" in native.last_error()
+
+
+def test_c_abi_rejects_a_tile_count_beyond_32_bits(native):
+    """The streaming kernels count the 32-key tiles of all (slot, kv head) pairs in 32 bits; the host refuses what
+    could overflow that before anything is launched (the pointers are never dereferenced on the host)."""
+    lib = native.load()
+    a = native.AttnArgs()
+    for name in ("q", "k_cache", "v_cache", "o", "time_dim_sizes", "user_phase"):
+        setattr(a, name, 256)
+    a.B, a.H, a.G, a.Tq, a.D, a.KV_CTX = 60000, 40000, 40000, 1, 8, 1 << 20
+    a.ctx_window_size, a.phase, a.stage, a.scale = 1 << 20, 2, 3, 1.0
+    a.q_stride = (ctypes.c_int64 * 4)(8, 8, 8, 1)
+    a.o_stride = (ctypes.c_int64 * 4)(8, 8, 8, 1)
+    a.k_stride_b = a.v_stride_b = 40000 * (1 << 20) * 8
+    a.time_dim_sizes_stride = a.user_phase_stride = 1
+    assert lib.g4b_attn_forward(ctypes.byref(a), None) == native.G4B_ERR_UNSUPPORTED
+    assert "2^31" in native.last_error()
+    a.B, a.G, a.H = 4, 2, 8
+    a.k_stride_b = a.v_stride_b = 2 * (1 << 20) * 8
+    a.q_dtype = 7  # the next check in line fails instead: the tile count passed
+    assert lib.g4b_attn_forward(ctypes.byref(a), None) == native.G4B_ERR_INVALID_ARGUMENT

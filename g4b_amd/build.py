@@ -3,6 +3,7 @@
     python -m g4b_amd.build            # compile every translation unit, link
     python -m g4b_amd.build --verbose  # also print the per-kernel register / LDS usage remarks
     python -m g4b_amd.build --check-waits  # also verify that nothing foreign sits in the hand-counted wait regions
+    python -m g4b_amd.build --asan     # host code of the C ABI under AddressSanitizer + UBSan (no GPU needed), and run it
 
 The shared library lands next to this file so that it travels with the source tree; nothing
 is installed.  hipcc cross-compiles for gfx950 without a GPU present.
@@ -104,8 +105,13 @@ def check_wait_discipline() -> dict:
                 end = next(j for j in range(i, len(lines)) if lines[j].startswith(".Lfunc_end"))
                 body = lines[i:end]
                 mfma = [j for j, l in enumerate(body) if "v_mfma" in l]
-                # A foreign access is harmless only if both counters are drained again before the next MFMA (the
-                # epilogue of a workgroup's first query tile and the set-up of its second sit between two MFMAs).
+                # A foreign access is harmless only if its counter is drained again before the next MFMA (the epilogue
+                # of a workgroup's first query tile and the set-up of its second sit between two MFMAs).  Every
+                # hand-counted wait stands directly in front of the MFMA that consumes what it waited for, so a wait
+                # that counted next to a foreign access is caught at that MFMA; a wait whose MFMA comes only after the
+                # drain has, by then, everything it counted on.  (The epilogue's own LDS traffic and the waits the
+                # compiler counts for it use the same mnemonics as the operand reads and cannot be told apart here.)
+                # A flat access holds a slot of both counters until it has completed, i.e. until vmcnt(0).
                 dirty_lgkm = dirty_vm = None
                 for l in body[mfma[0] : mfma[-1] + 1]:
                     ins = l.strip()
@@ -113,10 +119,12 @@ def check_wait_discipline() -> dict:
                         if dirty_lgkm or dirty_vm:
                             raise RuntimeError(f"{m.group(1)}: `{dirty_lgkm or dirty_vm}` inside the hand-counted wait region")
                     elif ins.startswith("s_waitcnt"):
-                        if "lgkmcnt(0)" in ins:
+                        if "lgkmcnt(0)" in ins and not (dirty_lgkm or "").startswith("flat_"):
                             dirty_lgkm = None
                         if "vmcnt(0)" in ins:
                             dirty_vm = None
+                            if (dirty_lgkm or "").startswith("flat_"):
+                                dirty_lgkm = None
                     elif foreign.search(ins) and not ins.startswith(allowed):
                         if ins.startswith(("s_load", "s_buffer_load", "ds_", "flat_")):
                             dirty_lgkm = ins
@@ -172,7 +180,40 @@ def check_stream_loads() -> dict:
     return {k: tuple(v) for k, v in seen.items()}
 
 
+# The host pass under AddressSanitizer and UndefinedBehaviorSanitizer (GPU sanitizers are not available here): the C ABI's
+# entry points and their validation (api.hip) linked with tests/host_api_check.hip, whose stand-in launchers abort, and
+# the share-out arithmetic of tests/tile_shares_check.hip.  Returns the two executables; they need no GPU.
+SANITIZE = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-Xarch_host", "-fno-sanitize-recover=undefined",
+            "-Xarch_host", "-fno-omit-frame-pointer", "-g"]
+
+
+def build_asan() -> list[Path]:
+    out_dir = BUILD_DIR / "asan"
+    out_dir.mkdir(parents=True, exist_ok=True)
+    tests = PKG_DIR.parent / "tests"
+    flags = ["-O1", "-std=c++17", "-fPIE", f"--offload-arch={ARCH}", "-Wno-inline-asm", "-Wno-unknown-pragmas", *DEVICE_FLAGS, *SANITIZE]
+
+    def run(cmd):
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"{' '.join(map(str, cmd[:3]))} ... failed:\n{res.stderr[-3000:]}")
+
+    api_check = out_dir / "host_api_check"
+    run([hipcc(), *flags, "-I", str(CSRC), str(CSRC / "api.hip"), str(tests / "host_api_check.hip"), "-o", str(api_check)])
+    shares_check = out_dir / "tile_shares_check"
+    run([hipcc(), *flags, "-I", str(CSRC), str(tests / "tile_shares_check.hip"), "-o", str(shares_check)])
+    return [api_check, shares_check]
+
+
 if __name__ == "__main__":
+    if "--asan" in sys.argv:
+        for exe in build_asan():
+            res = subprocess.run([str(exe)], capture_output=True, text=True, env=dict(os.environ, ASAN_OPTIONS="detect_leaks=0"))
+            print(f"{exe.name}: exit {res.returncode}: {(res.stdout.strip().splitlines() or [''])[-1]}")
+            if res.returncode:
+                print(res.stderr[-3000:], file=sys.stderr)
+                sys.exit(1)
+        sys.exit(0)
     path = build(verbose="--verbose" in sys.argv)
     print(path)
     if "--check-waits" in sys.argv:

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -18,6 +19,20 @@
 // per-device pointer that static_scratch_ptr() obtains with hipGetSymbolAddress.
 constexpr size_t kStaticScratchBytes = (size_t)G4B_ATTN_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Which XCD the workgroups of a launch run on.  The streaming kernels give the workers on even XCDs a larger share
+// (the odd ones stream from HBM more slowly), which only helps while workgroup i of a grid runs on an XCD of the parity
+// of i; nothing documents that order, so it is read from the hardware once per device: 64 workgroups write the XCC id
+// their wave reports (HW_REG_XCC_ID), the host looks at the parities.
+constexpr int kXcdProbeGroups = 64;
+static __device__ int32_t xcd_probe_ids[kXcdProbeGroups];
+__global__ void xcd_probe_kernel(int32_t* ids) {
+    if (threadIdx.x == 0) {
+        uint32_t x;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(x));
+        ids[blockIdx.x] = (int32_t)x;
+    }
+}
 
 namespace {
 
@@ -73,6 +88,66 @@ bool claim_static_scratch(hipStream_t stream) {
     return true;
 }
 
+// Environment switches, read once (the reference has G4B_FA_FORCE_CONFIG and G4B_FA_PRINT_CONFIG for an engine whose
+// call sites cannot be changed, g4b/kernels/fa2.py:148-150,691-700):
+//   G4B_ATTN_NUM_WORKERS=n   worker count of decode-shaped launches that pass num_workers = 0 (also sizes the workspace)
+//   G4B_ATTN_XCD_SHARES=0|1  0: equal shares for all workers; 1: the weighted shares without asking the hardware
+//   G4B_ATTN_PRINT_PLAN=1    one line on stderr per attention launch: kernel family, grid, workers, key splits
+struct EnvSwitches {
+    int num_workers = 0;
+    int xcd_shares = -1;  // -1: ask the hardware
+    bool print_plan = false;
+    EnvSwitches() {
+        if (const char* v = getenv("G4B_ATTN_NUM_WORKERS")) {
+            const long n = strtol(v, nullptr, 10);
+            if (n >= 1 && n <= (1 << 20)) num_workers = (int)n;
+        }
+        if (const char* v = getenv("G4B_ATTN_XCD_SHARES")) xcd_shares = (v[0] == '0') ? 0 : 1;
+        if (const char* v = getenv("G4B_ATTN_PRINT_PLAN")) print_plan = v[0] != '\0' && v[0] != '0';
+    }
+};
+const EnvSwitches& env_switches() {
+    static const EnvSwitches e;
+    return e;
+}
+
+// 1 when workgroup i of a grid runs on an XCD of the parity of i on the current device, else 0.  Asked once per device,
+// by the first launch that wants to know outside stream capture (it waits for the 64-workgroup probe: the one place
+// where this library synchronises); launches recorded into a graph before that are told 0 and keep equal shares.
+enum : int { XCD_UNKNOWN = 0, XCD_PARITY = 1, XCD_OTHER = 2 };
+int g_xcd_state[kMaxDevices] = {};
+int32_t g_xcd_ids[kMaxDevices][kXcdProbeGroups];
+int xcd_parity_known(hipStream_t stream) {
+    const EnvSwitches& env = env_switches();
+    if (env.xcd_shares >= 0) return env.xcd_shares;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_xcd_state[dev] != XCD_UNKNOWN) return g_xcd_state[dev] == XCD_PARITY;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) return 0;
+    void* ids = nullptr;
+    int state = XCD_OTHER;
+    if (hipGetSymbolAddress(&ids, HIP_SYMBOL(xcd_probe_ids)) == hipSuccess && ids) {
+        hipLaunchKernelGGL(xcd_probe_kernel, dim3(kXcdProbeGroups), dim3(64), 0, stream, static_cast<int32_t*>(ids));
+        if (hipGetLastError() == hipSuccess &&
+            hipMemcpyAsync(g_xcd_ids[dev], ids, sizeof(g_xcd_ids[dev]), hipMemcpyDeviceToHost, stream) == hipSuccess &&
+            hipStreamSynchronize(stream) == hipSuccess) {
+            state = XCD_PARITY;
+            for (int i = 0; i < kXcdProbeGroups; ++i)
+                if ((g_xcd_ids[dev][i] & 1) != (i & 1)) state = XCD_OTHER;
+        }
+    }
+    if (state == XCD_OTHER) (void)hipGetLastError();
+    g_xcd_state[dev] = state;
+    if (env.print_plan) {
+        fprintf(stderr, "g4b_attn: XCC ids of workgroups 0..15 on device %d:", dev);
+        for (int i = 0; i < 16; ++i) fprintf(stderr, " %d", g_xcd_ids[dev][i]);
+        fprintf(stderr, " -> %s shares\n", state == XCD_PARITY ? "weighted" : "equal");
+    }
+    return state == XCD_PARITY;
+}
+
 // g4b_profile_begin .. g4b_profile_end: one (start, stop) event pair per timed call of this thread
 thread_local bool g_profiling = false;
 thread_local std::vector<std::pair<hipEvent_t, hipEvent_t>> g_profile_records;
@@ -109,7 +184,10 @@ int fail(int code, const char* fmt, ...) {
 
 constexpr int kDefaultWorkers = 1024;  // 256 CUs x 4 SIMDs x 1 wave
 // a worker for head dimension 512 is a workgroup of two waves
-int default_workers(int D) { return D > 256 ? kDefaultWorkers * 256 / D : kDefaultWorkers; }
+int default_workers(int D) {
+    if (env_switches().num_workers > 0) return env_switches().num_workers;
+    return D > 256 ? kDefaultWorkers * 256 / D : kDefaultWorkers;
+}
 constexpr int kMaxDecodeRows = 16;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -195,7 +273,7 @@ int g4b_profile_end(float* ms, int32_t capacity) {
     return n;
 }
 int32_t g4b_abi_version(void) { return G4B_ATTN_ABI_VERSION; }
-int32_t g4b_attn_default_workers(void) { return kDefaultWorkers; }
+int32_t g4b_attn_default_workers(void) { return default_workers(256); }
 
 uint64_t g4b_attn_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t Tq, int32_t D, int32_t num_workers) {
     if (B < 1 || H < 1 || G < 1 || Tq < 1 || D < 1 || H % G) return 0;
@@ -294,7 +372,7 @@ static int fill_attn_params(const g4b_attn_args* a, g4b::AttnParams& p) {
     // a query wider than the cache type: f32 over f16 / bf16, f16 over bf16
     const bool q_wider = a->q_dtype == G4B_DT_F32 || (a->q_dtype == G4B_DT_F16 && a->kv_dtype == G4B_DT_BF16);
     p.q_split = (a->use_fp32_dot && q_wider) ? 1 : 0;
-    p.xcd_shift = 0;  // the decode kernels proper have one worker per workgroup, and workgroup i runs on XCD i % 8
+    p.xcd_shift = -1;  // equal shares; the decode launch asks xcd_parity_known()
     return G4B_OK;
 }
 
@@ -305,6 +383,8 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
     hipError_t e;
     if (takes_generic_path(a)) {
         if ((int64_t)a->B * a->H * a->Tq > 0x7fffffffLL) return fail(G4B_ERR_UNSUPPORTED, "B * H * Tq must be below 2^31 on this path");
+        if (env_switches().print_plan)
+            fprintf(stderr, "g4b_attn plan: B=%d H=%d G=%d Tq=%d D=%d: plain fp32 kernel\n", a->B, a->H, a->G, a->Tq, a->D);
         if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = g4b::launch_attn_generic(p, a->D, a->kv_dtype, a->on_band_block, static_cast<hipStream_t>(stream));
     } else if (rows <= kMaxDecodeRows) {
@@ -321,6 +401,14 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
         } else {
             p.NW = 0;  // one wave per (slot, kv head), no partials
         }
+        // the decode kernels proper have one worker per workgroup: weighted shares where workgroup i runs on an XCD of
+        // the parity of i
+        if (p.NW > 0 && xcd_parity_known(static_cast<hipStream_t>(stream))) p.xcd_shift = 0;
+        if (env_switches().print_plan)
+            fprintf(stderr, "g4b_attn plan: decode B=%d H=%d G=%d Tq=%d D=%d KV_CTX=%d W=%d: %s, %d workers, %s shares%s\n", a->B, a->H,
+                    a->G, a->Tq, a->D, a->KV_CTX, a->ctx_window_size,
+                    g4b::decode_pair_path(p, a->D) ? "one kernel, a workgroup per (slot, kv head)" : (p.NW > 0 ? "flat tile list + merge kernel" : "a wave per (slot, kv head)"),
+                    p.NW, p.xcd_shift >= 0 ? "weighted" : "equal", a->workspace ? "" : ", no workspace");
         if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = g4b::launch_attn_decode(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
     } else {
@@ -336,6 +424,11 @@ int g4b_attn_forward(const g4b_attn_args* a, void* stream) {
             p.part_o = static_cast<float*>(a->workspace);
             p.part_ml = prefill_partial_sums(a->workspace, p.split_slots, a->H, a->Tq, a->D);
         }
+        if (env_switches().print_plan)
+            fprintf(stderr, "g4b_attn plan: prefill B=%d H=%d G=%d Tq=%d D=%d KV_CTX=%d W=%d: grid %d, up to %d (slot, key split) pairs%s\n",
+                    a->B, a->H, a->G, a->Tq, a->D, a->KV_CTX, a->ctx_window_size,
+                    g4b::prefill_grid(p, a->D == 512 && p.q_split ? 64 : 128, a->D != 512), p.split_slots,
+                    p.pair_split ? ", pairs of query tiles cut into key spans" : "");
         if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
         e = a->D == 512 ? g4b::launch_attn_prefill_wide(p, a->kv_dtype, static_cast<hipStream_t>(stream))
                         : g4b::launch_attn_prefill(p, a->D, a->kv_dtype, static_cast<hipStream_t>(stream));
@@ -469,6 +562,7 @@ int g4b_static_scratch_init(void) {
     void* ptr = nullptr;
     const hipError_t e = static_scratch_ptr(&ptr);
     if (e != hipSuccess) return fail(G4B_ERR_LAUNCH, "static scratch: %s", hipGetErrorString(e));
+    (void)xcd_parity_known(nullptr);  // the other thing a launch may want to look up outside stream capture
     return G4B_OK;
 }
 
@@ -642,6 +736,7 @@ int g4b_rope(const g4b_rope_args* a, void* stream) {
     p.phase = a->phase;
     p.k_writeback = a->k_writeback;
     p.eps = a->rmsnorm_eps;
+    p.xcd_weighted = xcd_parity_known(static_cast<hipStream_t>(stream));
     if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
     hipError_t e = g4b::launch_rope(p, static_cast<hipStream_t>(stream));
     profile_disarm();

@@ -121,6 +121,7 @@ struct RopeParams {
     int32_t q_dt, k_dt, v_dt, cache_dt;
     int32_t B, H, G, t, D, Dv, T;
     int32_t phase, k_writeback;
+    int32_t xcd_weighted;  // 1: workgroup i of a grid runs on an XCD of the parity of i, and the even XCDs get 26 blocks of 50
     int32_t even_blocks;  // rope_kernel: token blocks dealt to the even workgroups (0: workgroup i takes token block i)
     float eps;
 };

@@ -174,7 +174,7 @@ hipError_t launch_rope(const RopeParams& p, hipStream_t stream) {
     int z = 1;
     while (z < 4 && z * 2 <= jobs && (int64_t)blocks * p.B * z < 256) z *= 2;
     RopeParams pk = p;
-    pk.even_blocks = blocks >= 128 ? (blocks * 26 + 49) / 50 : 0;
+    pk.even_blocks = (p.xcd_weighted && blocks >= 128) ? (blocks * 26 + 49) / 50 : 0;
     dim3 grid(pk.even_blocks ? 2 * pk.even_blocks : blocks, p.B, z);
     if (cpt == 4) G4B_LAUNCH_DOMINANT(rope_kernel<4>, grid, dim3(256), 0, stream, pk);
     else G4B_LAUNCH_DOMINANT(rope_kernel<8>, grid, dim3(256), 0, stream, pk);

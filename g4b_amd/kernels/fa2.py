@@ -113,6 +113,7 @@ def _bind(
     num_workers: int = 0,
     kernel_mask: int = 0,
     on_band_block: int | None = None,
+    limit_kv_splits: bool = False,
 ):
     """Validate the arguments like the reference and fill the C argument block (plus the objects it points into)."""
     assert isinstance(phase, int)  # fa2.py:653
@@ -152,6 +153,11 @@ def _bind(
         max_kv_splits = min(int(partial_o.shape[0]), int(partial_l.shape[0]), int(partial_m.shape[0]))  # fa2.py:658
 
     lib = _native.load()
+    if limit_kv_splits and max_kv_splits > 1 and (H // G) * Tq <= MAX_DECODE_ROWS:
+        # MAX_KV_SPLITS of the reference (fa2.py:658) as a bound: no more workers than max_kv_splits per (slot, kv head)
+        cap = B * G * max_kv_splits
+        default = int(lib.g4b_attn_default_workers()) * 256 // max(D, 256)  # a worker at head dimension 512 is two waves
+        num_workers = min(num_workers or default, cap)
     a = _native.AttnArgs()
     a.q, a.k_cache, a.v_cache, a.o = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr()
     a.time_dim_sizes, a.user_phase = time_dim_sizes.data_ptr(), user_phase.data_ptr()
@@ -240,6 +246,7 @@ def flash_attention(
     num_workers: int = 0,
     kernel_mask: int = 0,
     on_band_block: int | None = None,
+    limit_kv_splits: bool = False,
     stream=None,
     decode_q=None,
     decode_o=None,
@@ -302,7 +309,7 @@ def flash_attention(
         use_grouped_query_tile=use_grouped_query_tile, warp_specialize=warp_specialize, is_hopper=is_hopper,
         use_fp32_dot=use_fp32_dot, stage=stage, scale=scale, query_window=query_window, window_sizes=window_sizes,
         workspace=workspace, num_workers=num_workers, kernel_mask=kernel_mask, on_band_block=on_band_block,
-        decode_q=decode_q, decode_o=decode_o, decode_phase=decode_phase,
+        limit_kv_splits=limit_kv_splits, decode_q=decode_q, decode_o=decode_o, decode_phase=decode_phase,
     )
     _launch(entry, C.byref(a), C.c_void_p(U.current_stream() if stream is None else U.stream_handle(stream)), workspace is None)
     return None, None

@@ -7,7 +7,15 @@
  *   - Every pointer is a device pointer owned by the caller; the library never allocates,
  *     frees or synchronises (the scratch of g4b_attn_forward_static_scratch is an array in the
  *     library's device image, not an allocation).  Work is enqueued on `stream` (a hipStream_t passed as void*;
- *     NULL = the default stream) and is legal inside stream capture.
+ *     NULL = the default stream) and is legal inside stream capture.  One exception, once per GPU: the first
+ *     decode-shaped attention or rope launch (or g4b_static_scratch_init) outside stream capture runs a 64-workgroup
+ *     kernel that reports which XCD each workgroup ran on and waits for it on `stream`; the streaming kernels weight
+ *     their work shares by the answer.  Launches captured before that keep equal shares.
+ *   - Environment switches, read when the library is first used (counterparts of the reference's
+ *     G4B_FA_FORCE_CONFIG / G4B_FA_PRINT_CONFIG, g4b/kernels/fa2.py:148-150,691-700): G4B_ATTN_NUM_WORKERS=n sets the
+ *     default worker count of decode-shaped launches (and the size g4b_attn_workspace_bytes reports for it);
+ *     G4B_ATTN_XCD_SHARES=0 forces equal work shares, =1 the weighted ones without asking the hardware;
+ *     G4B_ATTN_PRINT_PLAN=1 prints one line per attention launch on stderr (kernel family, grid, workers, splits).
  *   - Strides are in ELEMENTS, as in the reference's launch adapter (g4b/kernels/utils.py:87-127).
  *   - Entry points return G4B_OK (0) or a negative g4b_status.  Arguments are validated on the
  *     host before anything is launched; g4b_last_error() returns a thread-local message for the

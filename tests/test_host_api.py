@@ -307,3 +307,20 @@ def test_c_abi_rejects_a_tile_count_beyond_32_bits(native):
     a.k_stride_b = a.v_stride_b = 2 * (1 << 20) * 8
     a.q_dtype = 7  # the next check in line fails instead: the tile count passed
     assert lib.g4b_attn_forward(ctypes.byref(a), None) == native.G4B_ERR_INVALID_ARGUMENT
+
+
+def test_limit_kv_splits_turns_the_partials_leading_dimension_into_a_bound(native):
+    """The reference's MAX_KV_SPLITS (fa2.py:658) does not bound the split by default; with limit_kv_splits=True a
+    decode launch gets at most that many workers per (slot, kv head)."""
+    from g4b_amd.kernels import fa2
+
+    q, k, v, o, tds, ph = _decode_args()
+    parts = (torch.zeros(4, 2, 8, 1, 256, dtype=torch.float16), torch.zeros(4, 2, 8, 1), torch.zeros(5, 2, 8, 1))
+    a, _, _ = fa2._bind(q, k, v, o, tds, ph, 64, 2, *parts, workspace=False)
+    assert a.num_workers == 0
+    a, _, _ = fa2._bind(q, k, v, o, tds, ph, 64, 2, *parts, workspace=False, limit_kv_splits=True)
+    assert a.num_workers == 2 * 2 * 4  # B * G * min of the leading dimensions
+    a, _, _ = fa2._bind(q, k, v, o, tds, ph, 64, 2, *parts, workspace=False, limit_kv_splits=True, num_workers=7)
+    assert a.num_workers == 7
+    a, _, _ = fa2._bind(q, k, v, o, tds, ph, 64, 2, workspace=False, limit_kv_splits=True)  # no partials: no bound
+    assert a.num_workers == 0

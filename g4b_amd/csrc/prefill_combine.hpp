@@ -7,7 +7,10 @@ namespace g4b {
 // Merge the key splits of a prefill-shaped launch: a lane per four output columns of a row, PFC_ROWS rows per
 // workgroup, every load of a row independent of the others.
 constexpr int PFC_ROWS = 8;
-template <int D, int NS, class T>
+// SPANS: the launch cut pairs of query tiles into key spans (AttnParams::pair_split): a split may have no rows for a
+// query tile, or have written them straight to o, and says so in its sums.  Otherwise every split has written its
+// rows, and their loads are issued with the loads of the sums instead of behind them: one round trip to memory less.
+template <int D, int NS, class T, bool SPANS>
 G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, int tb, int nsplit) {
     constexpr int LPR = D / 4;      // lanes per row
     constexpr int RPP = 256 / LPR;  // rows per pass
@@ -26,13 +29,14 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
             ls[s] = (s < nsplit) ? p.part_ml[prow * 2 + 1] : 0.f;
             final_row |= ls[s] < 0.f;
         }
-        if (final_row) continue;
+        if constexpr (SPANS)
+            if (final_row) continue;
         // spans without key tiles of the row's query tile left (0, 0) and no sums: only what was written is read
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             const int64_t prow = ((int64_t)(a_idx * nsplit + min(s, nsplit - 1)) * p.H + h) * p.Tq + t;
             const f4 zero = {0.f, 0.f, 0.f, 0.f};
-            if (ls[s] > 0.f) {
+            if (SPANS ? ls[s] > 0.f : s < nsplit) {
                 float x[4];
                 load_f32<4>(p.part_o, prow * D + d0, T::dt, x);
                 ov[s] = f4{x[0], x[1], x[2], x[3]};
@@ -80,13 +84,18 @@ G4B_DEV void prefill_combine_body(const AttnParams& p, const int bid, int* sh_sc
     const int nsplit = prefill_splits(p.split_slots, n_active);
     if (b < 0 || nsplit == 1) return;
     if (nsplit <= 2) {
-        prefill_combine_rows<D, 2, T>(p, a_idx, b, h, tb, nsplit);
+        if (p.pair_split) prefill_combine_rows<D, 2, T, true>(p, a_idx, b, h, tb, nsplit);
+        else prefill_combine_rows<D, 2, T, false>(p, a_idx, b, h, tb, nsplit);
     } else if constexpr (NSMAX >= 4) {
         if (nsplit <= 4) {
-            prefill_combine_rows<D, 4, T>(p, a_idx, b, h, tb, nsplit);
+            if (p.pair_split) prefill_combine_rows<D, 4, T, true>(p, a_idx, b, h, tb, nsplit);
+            else prefill_combine_rows<D, 4, T, false>(p, a_idx, b, h, tb, nsplit);
         } else if constexpr (NSMAX >= 8) {
-            if (nsplit <= 8) prefill_combine_rows<D, 8, T>(p, a_idx, b, h, tb, nsplit);
-            else if constexpr (NSMAX >= 16) prefill_combine_rows<D, 16, T>(p, a_idx, b, h, tb, nsplit);
+            if (nsplit <= 8) {
+                if (p.pair_split) prefill_combine_rows<D, 8, T, true>(p, a_idx, b, h, tb, nsplit);
+                else prefill_combine_rows<D, 8, T, false>(p, a_idx, b, h, tb, nsplit);
+            }
+            else if constexpr (NSMAX >= 16) prefill_combine_rows<D, 16, T, false>(p, a_idx, b, h, tb, nsplit);  // (pairs are cut into five spans at most)
         }
     }
 }

@@ -546,7 +546,7 @@ int g4b_attn_forward_mixed(const g4b_attn_args* prefill, const g4b_attn_args* de
     }
     g4b::MixedPlan mp = m.plan;
     mp.npx = (g4b::prefill_grid(pp, pf_rows, a->D != 512) + 7) / 8;
-    mp.combine_pf = g4b::prefill_combine_grid(pp);
+    mp.combine_pf = g4b::prefill_combine_blocks(pp, a->D);
     mp.combine_dec = (pair || !m.nw) ? 0 : a->B * a->G * pd.R * pd.Tq;
     if (!profile_arm()) return fail(G4B_ERR_LAUNCH, "could not create profiling events");
     const hipStream_t st = static_cast<hipStream_t>(stream);

@@ -52,7 +52,8 @@ __global__ __launch_bounds__(256) void attn_mixed_combine(const AttnParams pp, c
     __shared__ int sh_scan[8];
     __shared__ DecodeCombineSmem<D> sm;
     if ((int)blockIdx.x < mp.combine_pf) {
-        prefill_combine_body<D, T>(pp, blockIdx.x, sh_scan);
+        const int tblocks = (pp.Tq + pfc_rows(D) - 1) / pfc_rows(D);
+        prefill_combine_body<D, T>(pp, blockIdx.x % tblocks, (blockIdx.x / tblocks) % pp.H, blockIdx.x / (tblocks * pp.H), sh_scan);
         return;
     }
     const int d = blockIdx.x - mp.combine_pf, rows = pd.R * pd.Tq;

@@ -32,7 +32,6 @@
 
 namespace g4b {
 
-constexpr int PF_BN = 64;      // keys per tile
 constexpr int PF_PD = 6;       // LDS operand fetches in flight (issued and retired in pairs)
 
 template <int D>
@@ -131,24 +130,12 @@ G4B_DEV void prefill_body(const AttnParams& p, const int bid, char* smem, int* s
             tile_span(qtile_first, n_first);
             if (n_items == 2) tile_span(qtile_second, n_second);
         }
-        // Spans of equal cost, not of equal length: a query tile costs a workgroup about four key tiles' time besides
-        // its key tiles (staging, Q, first scores, epilogue), and the span in which the list passes from the first
-        // query tile to the second pays that twice.  With equal lengths the workgroups of that span finished 12 % after
-        // the others (S = 4096: 101 against 89 us).
-        constexpr int ITEM_COST = 4;
-        const int n_all = n_first + n_second;
-        const int target = (n_all + ITEM_COST * (nsplit + 1) + nsplit - 1) / nsplit;
-        int pos = 0;
-        for (int k = 0; k < nsplit; ++k) {  // the same walk in every workgroup of the pair
-            int end = pos + target - ITEM_COST;
-            if (pos < n_first && end > n_first && n_second > 0) end = max(end - ITEM_COST, n_first);
-            end = (k == nsplit - 1) ? n_all : min(max(end, pos), n_all);
+        pf_pair_spans(n_first, n_second, nsplit, [&](int k, int begin, int end) {  // the same walk in every workgroup of the pair
             if (k == split) {
-                span0 = pos;
+                span0 = begin;
                 span1 = end;
             }
-            pos = end;
-        }
+        });
     }
 
     const char* kbase = static_cast<const char*>(p.k) + ((int64_t)b * p.k_sb + (int64_t)g * KV_CTX * D) * 2;

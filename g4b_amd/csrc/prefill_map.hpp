@@ -5,6 +5,7 @@
 namespace g4b {
 
 constexpr int PF_BM = 128;     // query rows per workgroup
+constexpr int PF_BN = 64;      // keys per tile of the 128 / 256 kernel
 constexpr float PF_TAU = 8.f;  // log2 of the growth of a row maximum that triggers a rescale
 
 // Linear workgroup id -> (head, query tile rank).  "Heads" are (active slot, kv head, key split) triples.  Workgroups
@@ -65,6 +66,36 @@ __host__ __device__ inline int pf_items_per_workgroup(int nsplit, int nq, bool p
 // Ranks (workgroups) per head: query tiles, or pairs of them.
 __host__ __device__ inline int pf_ranks(int nsplit, int nq, bool pair_split, int unsplit_heads) {
     return pf_items_per_workgroup(nsplit, nq, pair_split, unsplit_heads) == 2 ? (nq + 1) / 2 : nq;
+}
+
+// The spans of a pair's key-tile list (pair_split): n_first tiles of the first query tile, then n_second of the second,
+// cut into nsplit spans; visit(k, begin, end) is called for span k = 0 .. nsplit - 1 in order.  Spans of equal cost,
+// not of equal length: a query tile costs a workgroup about four key tiles' time besides its key tiles (staging, Q,
+// first scores, epilogue), and the span in which the list passes from the first query tile to the second pays that
+// twice.  With equal lengths the workgroups of that span finished 12 % after the others (S = 4096: 101 against 89 us;
+// costs of 3, 5, 6 and 8 tiles measured worse).
+constexpr int PF_ITEM_COST = 4;
+template <class Visit>
+__host__ __device__ inline void pf_pair_spans(int n_first, int n_second, int nsplit, Visit&& visit) {
+    const int n_all = n_first + n_second;
+    const int target = (n_all + PF_ITEM_COST * (nsplit + 1) + nsplit - 1) / nsplit;
+    int pos = 0;
+    for (int k = 0; k < nsplit; ++k) {
+        int end = pos + target - PF_ITEM_COST;
+        if (pos < n_first && end > n_first && n_second > 0) end = end - PF_ITEM_COST > n_first ? end - PF_ITEM_COST : n_first;
+        end = end > pos ? end : pos;
+        end = (k == nsplit - 1 || end > n_all) ? n_all : end;
+        visit(k, pos, end);
+        pos = end;
+    }
+}
+// What a span [begin, end) of that list does for the query tile whose key tiles are [base, base + n) of it: 2 = it
+// holds all of them (the rows are final and go straight to o), 1 = some (partial rows are written), 0 = none.
+__host__ __device__ inline int pf_span_part(int begin, int end, int base, int n) {
+    if (n <= 0) return 0;
+    if (begin <= base && end - base >= n) return 2;
+    const int first = begin - base > 0 ? begin - base : 0, last = (end - base < n ? end - base : n) - 1;
+    return last >= first ? 1 : 0;
 }
 
 // Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on

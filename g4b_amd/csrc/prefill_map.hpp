@@ -89,15 +89,6 @@ __host__ __device__ inline void pf_pair_spans(int n_first, int n_second, int nsp
         pos = end;
     }
 }
-// What a span [begin, end) of that list does for the query tile whose key tiles are [base, base + n) of it: 2 = it
-// holds all of them (the rows are final and go straight to o), 1 = some (partial rows are written), 0 = none.
-__host__ __device__ inline int pf_span_part(int begin, int end, int base, int n) {
-    if (n <= 0) return 0;
-    if (begin <= base && end - base >= n) return 2;
-    const int first = begin - base > 0 ? begin - base : 0, last = (end - base < n ? end - base : n) - 1;
-    return last >= first ? 1 : 0;
-}
-
 // Grid for the worst case over the number of slots that turn out to be in phase; the kernels read that number on
 // the device and surplus workgroups leave at once.  paired: the kernel gives a workgroup pf_items_per_workgroup tiles.
 inline int prefill_grid(const AttnParams& p, int bm = PF_BM, bool paired = true) {

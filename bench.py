@@ -293,7 +293,7 @@ class Prefill(Workload):
 
     bound = "mfma"
 
-    def __init__(self, device, S, query_window=None, seed=0, dim=D, bf16=False):
+    def __init__(self, device, S, query_window=None, seed=0, dim=D, bf16=False, engine_call=False):
         import torch
 
         from g4b_amd.kernels import fa2
@@ -307,10 +307,18 @@ class Prefill(Workload):
         dt = torch.bfloat16 if bf16 else torch.float16
         if bf16:
             self.name += "_bf16"
-        self.q = _randn_f16((1, H, S, D_), seed + 1, device, dt)
+        self.engine_call = engine_call
+        if engine_call:
+            # what the engine passes (gemma4e.py:593-607): fp32 q and o as [B, H, t, D] views of [B, t, H, D] scratchpads,
+            # use_fp32_dot=True, so q enters K Q^T as a pair of 16-bit operands
+            self.name += "_fp32q"
+            self.q = _randn_f16((1, S, H, D_), seed + 1, device, torch.float32).permute(0, 2, 1, 3)
+            self.o = torch.empty((1, S, H, D_), dtype=torch.float32, device=device).permute(0, 2, 1, 3)
+        else:
+            self.q = _randn_f16((1, H, S, D_), seed + 1, device, dt)
+            self.o = torch.empty_like(self.q)
         self.k = _randn_f16((1, G, S, D_), seed + 2, device, dt)
         self.v = _randn_f16((1, G, S, D_), seed + 3, device, dt)
-        self.o = torch.empty_like(self.q)
         self.tds = torch.full((1,), S, dtype=torch.int32, device=device)
         self.phase = torch.full((1,), fa2.PHASE_PREFILL, dtype=torch.uint8, device=device)
         if query_window is None:
@@ -323,14 +331,14 @@ class Prefill(Workload):
         need = fa2.workspace_bytes(1, H, G, S, D_)
         self.ws = torch.empty(need, dtype=torch.uint8, device=device) if need and WORKSPACE_MODE == "caller" else None
         self.flops = 4 * H * D_ * pairs
-        self.bytes = (2 * H * S * D_ + 2 * G * S * D_) * 2
+        self.bytes = 2 * H * S * D_ * (4 if engine_call else 2) + 2 * G * S * D_ * 2
         self.units = self.flops
 
     def launch(self, i=0, kernel_mask=0):
         if self.plan is None:
             self.plan = self.fa2.plan_flash_attention(
                 self.q, self.k, self.v, self.o, self.tds, self.phase, self.S, self.fa2.PHASE_PREFILL,
-                scale=SCALE, query_window=self.qw, workspace=WORKSPACE_OF(self.ws),
+                scale=SCALE, query_window=self.qw, workspace=WORKSPACE_OF(self.ws), use_fp32_dot=self.engine_call,
             )
         self.plan.launch()
 
@@ -493,6 +501,9 @@ WORKLOADS = {
     "prefill_swa_8192": lambda dev: Prefill(dev, 8192, query_window=512),
     "prefill_causal_8192_d512": lambda dev: Prefill(dev, 8192, dim=512),
     "prefill_causal_8192_bf16": lambda dev: Prefill(dev, 8192, bf16=True),
+    # the engine's own call: fp32 q / o scratchpads in token-major layout, use_fp32_dot=True (flops counted as for fp16 q)
+    "prefill_causal_8192_fp32q": lambda dev: Prefill(dev, 8192, engine_call=True),
+    "prefill_causal_8192_d512_fp32q": lambda dev: Prefill(dev, 8192, dim=512, engine_call=True),
     "mixed_step": lambda dev: MixedStep(dev),
     "mixed_step_two_launches": lambda dev: MixedStep(dev, one_launch=False),
     # the same step with Gemma-4's layer shapes: head dimension 256 on sliding-window layers, 512 on global ones
@@ -783,7 +794,7 @@ def main():
             torch.cuda.empty_cache()
 
     primary_is_hbm = res["roofline"]["bound"] == "hbm"
-    head_dim = 512 if args.workload.endswith("_d512") else D
+    head_dim = 512 if "_d512" in args.workload else D
     line = {
         "metric": METRIC,
         "value": round(res["GBps"] if primary_is_hbm else res["TFLOPs"], 2),

@@ -15,9 +15,11 @@
 //
 // QS (a query wider than the cache type, to enter K Q^T unrounded): there is no register left for a second Q block,
 // so a wave owns 16 rows and the 32 columns of its B operand hold their rounded values (columns 0..15) and their
-// rounding errors (columns 16..31).  The two halves of S^T are added across the lane pair (n, n + 16) right after the
-// first product, which leaves both lanes with the score of the unrounded query; from there on the lanes of a pair
-// carry the same row (the second product computes it twice) and a workgroup covers 64 rows.
+// rounding errors (columns 16..31); a workgroup covers 64 rows.  The two halves of S^T are added across the lane pair
+// (n, n + 16) right after the first product, each lane of the pair keeping the sums of 16 of the tile's 32 keys: the
+// four lanes of a row (n, n + 16, n + 32, n + 48) then hold eight keys each, which is the B operand of
+// v_mfma_f32_16x16x32 -- the second product runs on 16-column tiles (32 MFMAs of half the cycles, accumulators in
+// 128 registers) instead of computing every row twice on 32-column ones, and the softmax handles every score once.
 #pragma once
 #include "common.hpp"
 #include "prefill_combine.hpp"
@@ -39,6 +41,20 @@ G4B_DEV float row16_pair_sum(float x) {
     const uint32_t b = __builtin_bit_cast(uint32_t, x);
     const u2 r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
     const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+G4B_DEV float row16_pair_max(float x) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    const u2 r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+// a of the even 16-lane rows plus the pair lane's a, b of the odd rows plus the pair lane's b: lane l of an even row
+// receives a(l) + a(l + 16), lane l + 16 receives b(l) + b(l + 16).
+G4B_DEV float row16_pair_sum_split(float a, float b) {
+    const u2 r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
+    const uint32_t r0 = r[0], r1 = r[1];  // (a.row0, b.row0, a.row2, b.row2), (a.row1, b.row1, a.row3, b.row3)
     return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
 }
 
@@ -81,11 +97,17 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
     if (row_ok) row_range(p, si, ti, lo_r, hi_r);
     const int64_t qoff = (int64_t)b * p.q_s[0] + (int64_t)(g * R + hh) * p.q_s[1] + (int64_t)ti * p.q_s[2];
 
-    f16v acc[DT];  // 256 accumulator registers: the whole AGPR file
+    f16v acc[QS ? 1 : DT];  // 256 accumulator registers: the whole AGPR file
 #pragma unroll
-    for (int i = 0; i < DT; ++i)
+    for (int i = 0; i < (QS ? 1 : DT); ++i)
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+    // split query: O^T as 32 tiles of 16 d x 16 rows; lane (row n16, group kg = lane / 16) holds d = 16 blk + 4 kg + 0..3
+    constexpr int NB16 = D / 16;
+    f4 acc16[QS ? NB16 : 1];
+#pragma unroll
+    for (int i = 0; i < (QS ? NB16 : 1); ++i) acc16[i] = f4{0.f, 0.f, 0.f, 0.f};
+    const int n16 = lane & 15, u16 = (lane >> 4) & 1, kg = lane >> 4;
     float m_run = -INFINITY, l_run = 0.f;
 
     if (hi_wg > lo_wg) {
@@ -139,6 +161,17 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
             const int piece = d8 * 4 + tr_dhalf * 2 + (tr_q >> 1);
             voff[d8] = 2 * TILE + (uint32_t)tr_key * ROW + (uint32_t)((piece ^ (4 * (tr_key & 7))) * 16) + (uint32_t)(tr_q & 1) * 8u;
         }
+        // split query: V^T fragment of d tile blk for lane group kg: d = 16 blk + n16, keys {16 u16 + 4 h2 + 0..3, the same
+        // + 8}; the swizzle touches bits 1..3 of blk, blk / 16 becomes an instruction offset
+        uint32_t voff16[QS ? 16 : 1];
+        if constexpr (QS) {
+            const int key = 16 * u16 + tr_key;
+#pragma unroll
+            for (int bl = 0; bl < 16; ++bl) {
+                const int piece = 2 * bl + (tr_q >> 1);
+                voff16[bl] = 2 * TILE + (uint32_t)key * ROW + (uint32_t)((piece ^ (4 * (key & 7))) * 16) + (uint32_t)(tr_q & 1) * 8u;
+            }
+        }
         uint32_t stage_base = lds0;
         auto k_issue = [&](int c) -> u4 { return lds_read16(stage_base + koff[c & 7], (c >> 3) * 256); };
         struct VFrag {
@@ -149,6 +182,12 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
             VFrag f;
             f.lo = lds_read8_tr16(stage_base + voff[dt & 7], cu * 16 * ROW + (dt >> 3) * 512);
             f.hi = lds_read8_tr16(stage_base + voff[dt & 7], (cu * 16 + 8) * ROW + (dt >> 3) * 512);
+            return f;
+        };
+        auto v_issue16 = [&](int blk) -> VFrag {
+            VFrag f;
+            f.lo = lds_read8_tr16(stage_base + voff16[blk & 15], (blk >> 4) * 512);
+            f.hi = lds_read8_tr16(stage_base + voff16[blk & 15], 8 * ROW + (blk >> 4) * 512);
             return f;
         };
         auto wait_pair = [&](u4& a0, u4& a1, int left) {
@@ -223,59 +262,118 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
                     }
                 }
 
-                if constexpr (QS) {
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) s[j] = row16_pair_sum(s[j]);  // K q_hi + K q_lo
-                }
-
-                // ---- edge tiles: mask
                 const int jb = kt * PW_BN;
-                if ((jb < lo_max) || (jb + PW_BN > hi_min)) {
-                    pf_mask_block(s, jb, h2, lo_r, hi_r);
-                }
-
-                // ---- online softmax with lazy rescaling (the exponent reference moves only when the maximum outgrows
-                // it by more than 2^PF_TAU)
-                float mx = s[0];
+                if constexpr (QS) {
+                    // K q_hi + K q_lo: lane (n16, u16, h2) keeps score j of key jb + 16 u16 + 8 (j / 4) + 4 h2 + j % 4
+                    float t[8];
 #pragma unroll
-                for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
-                mx = half_swap_max(mx) * p.c;
-                G4B_PF_LAZY_RESCALE(acc, DT, m_run, l_run, mx);
-                const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
-                float psum = 0.f;
-                u4 pf[2];  // [16-key group] -> 8 keys of this lane half
+                    for (int j = 0; j < 8; ++j) {
+                        const float a = s[j], b8 = s[j + 8];
+                        t[j] = row16_pair_sum_split(a, b8);
+                    }
+                    if ((jb < lo_max) || (jb + PW_BN > hi_min)) {  // edge tiles: mask
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                        for (int j = 0; j < 8; ++j) {
+                            const int key = jb + 16 * u16 + 8 * (j >> 2) + 4 * h2 + (j & 3);
+                            if (key < lo_r || key >= hi_r) t[j] = -INFINITY;
+                        }
+                    }
+                    float mx = t[0];
+#pragma unroll
+                    for (int j = 1; j < 8; ++j) mx = fmaxf(mx, t[j]);
+                    mx = half_swap_max(row16_pair_max(mx)) * p.c;  // over the four lanes of the row
+                    {   // lazy rescaling (G4B_PF_LAZY_RESCALE for the 16-column accumulators)
+                        const bool grow = mx > m_run + PF_TAU;
+                        if (__any(grow)) {
+                            const float alpha = grow ? fast_exp2(m_run - mx) : 1.f;  // 0 on a row's first keys
+                            const bool touch = grow && (m_run != -INFINITY);
+                            m_run = grow ? mx : m_run;
+                            l_run *= alpha;
+                            if (__any(touch)) {
+#pragma unroll
+                                for (int i = 0; i < NB16; ++i) acc16[i] = acc16[i] * alpha;
+                            }
+                        }
+                    }
+                    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
                     float e[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) e[j] = fast_exp2(__builtin_fmaf(s[8 * u + j], p.c, -m_safe));
-                    pf[u] = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
+                    for (int j = 0; j < 8; ++j) e[j] = fast_exp2(__builtin_fmaf(t[j], p.c, -m_safe));
+                    const u4 pf = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
+                    float psum = 0.f;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const uint32_t w = pf[u][j];
+                        const uint32_t w = pf[j];
                         psum = T::sum2(w, psum);  // the row sum adds up the rounded values the second product uses
                     }
-                }
-                l_run += psum;
+                    l_run += psum;
 
-                // ---- O^T += V^T P
-                {
+                    // ---- O^T += V^T P on 16 x 16 tiles: lane group kg contracts its eight keys
                     VFrag vbuf[PW_PD];
 #pragma unroll
-                    for (int i = 0; i < PW_PD; ++i) vbuf[i] = v_issue(i);
+                    for (int i = 0; i < PW_PD; ++i) vbuf[i] = v_issue16(i);
 #pragma unroll
-                    for (int idx = 0; idx < PV_STEPS; idx += 2) {
+                    for (int idx = 0; idx < NB16; idx += 2) {
                         VFrag f0 = vbuf[idx % PW_PD], f1 = vbuf[(idx + 1) % PW_PD];
-                        wait_pair2(f0, f1, (PV_STEPS - 2 - idx) / 2);
-                        if (idx + PW_PD < PV_STEPS) {
-                            vbuf[idx % PW_PD] = v_issue(idx + PW_PD);
-                            vbuf[(idx + 1) % PW_PD] = v_issue(idx + 1 + PW_PD);
+                        wait_pair2(f0, f1, (NB16 - 2 - idx) / 2);
+                        if (idx + PW_PD < NB16) {
+                            vbuf[idx % PW_PD] = v_issue16(idx + PW_PD);
+                            vbuf[(idx + 1) % PW_PD] = v_issue16(idx + 1 + PW_PD);
                         }
-                        const int cu = idx / DT, dt = idx % DT;  // DT is even: both steps share the key group
                         const u4 a0 = {f0.lo[0], f0.lo[1], f0.hi[0], f0.hi[1]};
                         const u4 a1 = {f1.lo[0], f1.lo[1], f1.hi[0], f1.hi[1]};
-                        acc[dt] = T::mfma32(a0, pf[cu], acc[dt]);
-                        acc[dt + 1] = T::mfma32(a1, pf[cu], acc[dt + 1]);
+                        acc16[idx] = T::mfma16(a0, pf, acc16[idx]);
+                        acc16[idx + 1] = T::mfma16(a1, pf, acc16[idx + 1]);
+                    }
+                } else {
+                    // ---- edge tiles: mask
+                    if ((jb < lo_max) || (jb + PW_BN > hi_min)) {
+                        pf_mask_block(s, jb, h2, lo_r, hi_r);
+                    }
+
+                    // ---- online softmax with lazy rescaling (the exponent reference moves only when the maximum outgrows
+                    // it by more than 2^PF_TAU)
+                    float mx = s[0];
+#pragma unroll
+                    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+                    mx = half_swap_max(mx) * p.c;
+                    G4B_PF_LAZY_RESCALE(acc, DT, m_run, l_run, mx);
+                    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
+                    float psum = 0.f;
+                    u4 pf[2];  // [16-key group] -> 8 keys of this lane half
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        float e[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) e[j] = fast_exp2(__builtin_fmaf(s[8 * u + j], p.c, -m_safe));
+                        pf[u] = u4{T::pack2(e[0], e[1]), T::pack2(e[2], e[3]), T::pack2(e[4], e[5]), T::pack2(e[6], e[7])};
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const uint32_t w = pf[u][j];
+                            psum = T::sum2(w, psum);  // the row sum adds up the rounded values the second product uses
+                        }
+                    }
+                    l_run += psum;
+
+                    // ---- O^T += V^T P
+                    {
+                        VFrag vbuf[PW_PD];
+#pragma unroll
+                        for (int i = 0; i < PW_PD; ++i) vbuf[i] = v_issue(i);
+#pragma unroll
+                        for (int idx = 0; idx < PV_STEPS; idx += 2) {
+                            VFrag f0 = vbuf[idx % PW_PD], f1 = vbuf[(idx + 1) % PW_PD];
+                            wait_pair2(f0, f1, (PV_STEPS - 2 - idx) / 2);
+                            if (idx + PW_PD < PV_STEPS) {
+                                vbuf[idx % PW_PD] = v_issue(idx + PW_PD);
+                                vbuf[(idx + 1) % PW_PD] = v_issue(idx + 1 + PW_PD);
+                            }
+                            const int cu = idx / DT, dt = idx % DT;  // DT is even: both steps share the key group
+                            const u4 a0 = {f0.lo[0], f0.lo[1], f0.hi[0], f0.hi[1]};
+                            const u4 a1 = {f1.lo[0], f1.lo[1], f1.hi[0], f1.hi[1]};
+                            acc[dt] = T::mfma32(a0, pf[cu], acc[dt]);
+                            acc[dt + 1] = T::mfma32(a1, pf[cu], acc[dt + 1]);
+                        }
                     }
                 }
                 vm_wait_all();
@@ -286,7 +384,7 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
 
     // ---- epilogue: the wave turns its 32 x 512 block around in LDS, 256 columns at a time (32 KiB of the staging
     // area per wave, free after the loop's last barrier), and stores 1 KiB row halves
-    const float l_tot = half_swap_sum(l_run);
+    const float l_tot = QS ? half_swap_sum(row16_pair_sum(l_run)) : half_swap_sum(l_run);
     const bool partial = nsplit > 1;
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;  // a key split's rows are normalised too: they are kept in 16 bits
     char* wbase = smem + wave * (32 * 256 * 4);
@@ -314,15 +412,23 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
     }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
+        if constexpr (QS) {
 #pragma unroll
-        for (int d8 = 0; d8 < 8; ++d8)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const int dt = half * 8 + d8;
-                f4 v = {acc[dt][4 * q4] * inv, acc[dt][4 * q4 + 1] * inv, acc[dt][4 * q4 + 2] * inv, acc[dt][4 * q4 + 3] * inv};
-                const int pc = 8 * d8 + 2 * q4 + h2;
-                *reinterpret_cast<f4*>(wbase + n32 * 1024 + ((pc ^ (n32 & 15)) * 16)) = v;
+            for (int bl = 0; bl < 16; ++bl) {  // d = 256 half + 16 bl + 4 kg + 0..3: piece 4 bl + kg of the row's half
+                const int pc = 4 * bl + kg;
+                *reinterpret_cast<f4*>(wbase + n16 * 1024 + ((pc ^ n16) * 16)) = acc16[half * 16 + bl] * inv;
             }
+        } else {
+#pragma unroll
+            for (int d8 = 0; d8 < 8; ++d8)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const int dt = half * 8 + d8;
+                    f4 v = {acc[dt][4 * q4] * inv, acc[dt][4 * q4 + 1] * inv, acc[dt][4 * q4 + 2] * inv, acc[dt][4 * q4 + 3] * inv};
+                    const int pc = 8 * d8 + 2 * q4 + h2;
+                    *reinterpret_cast<f4*>(wbase + n32 * 1024 + ((pc ^ (n32 & 15)) * 16)) = v;
+                }
+        }
         // Rows go eight at a time, their LDS reads first and in one block; the type is chosen per batch and the rows of
         // a batch are one scalar offset plus a stride apart (a wave has its SIMD to itself here: row by row -- read,
         // wait, compute the offset, choose the type, convert, store -- every row paid the LDS latency and some thirty
@@ -330,7 +436,7 @@ G4B_DEV void prefill_wide_body(const AttnParams& p, const int bid, char* smem, i
         auto store_rows = [&](auto nt, const int dt) {
             constexpr bool NT = decltype(nt)::value;
 #pragma unroll 1
-            for (int r0 = 0; r0 < WROWS; r0 += 8) {  // with a split query the LDS rows 16..31 are copies of 0..15
+            for (int r0 = 0; r0 < WROWS; r0 += 8) {
                 f4 v[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j)  // 64 lanes x 16 bytes = 256 fp32 columns of one row

@@ -337,6 +337,23 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
         return;
     }
 
+    if (B == 1) {
+        // A single slot (single-sequence decode: a launch of a few microseconds that is all latency): its tile count is
+        // the whole list, so the sums and prefix sums over the slots and the search for the slot fall away.
+        const SlotInfo si = slot_info(p, 0);
+        const int tlb = slot_tiles(si);
+        const TileShares shares = tile_shares(p, G * tlb);
+        if (w >= shares.nw) return;  // (also: no tiles at all)
+        const int64_t ws = shares.begin(w), we = shares.begin(w + 1);
+        for (int g = (int)(ws / tlb); g < G && (int64_t)g * tlb < we; ++g) {
+            const int64_t fs = (int64_t)g * tlb;
+            const int t0 = (int)(max(ws, fs) - fs);
+            const int t1 = (int)(min(we, fs + tlb) - fs);
+            if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, si, w, 0, g, t0, t1, tlb, xch);
+        }
+        return;
+    }
+
     // ---- flat tile list: total, then this worker's range ------------------------------------
     // lane l keeps what it read of slot l (the first 64 slots) for the second pass and for the segments
     int total = 0, tl_first = 0;
@@ -471,7 +488,11 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
     // flat start of this pair and total tile count (same arithmetic as the workers), computed by every wave
     int before = 0, total = 0;
     SlotInfo si_first = {};  // lane l keeps what it read of slot l (the first 64 slots)
-    for (int b0 = 0; b0 < B; b0 += 64) {
+    if (B == 1) {  // a single slot: nothing to sum (the launch is all latency, and this is a dozen instructions of it)
+        si_first = slot_info(p, 0);
+        total = G * slot_tiles(si_first);
+    }
+    for (int b0 = 0; b0 < (B == 1 ? 0 : B); b0 += 64) {
         const int x = b0 + lane;
         int c = 0;
         if (x < B) {
@@ -482,10 +503,12 @@ G4B_DEV void decode_combine_body(const AttnParams& p, int pair, int row, DecodeC
         total += c;
         before += (x < b) ? c : 0;
     }
-    total = wave_sum_i(total);
-    before = wave_sum_i(before);
+    if (B > 1) {
+        total = wave_sum_i(total);
+        before = wave_sum_i(before);
+    }
 
-    const SlotInfo si = b < 64 ? slot_info_of_lane(si_first, b) : slot_info(p, b);
+    const SlotInfo si = B == 1 ? si_first : (b < 64 ? slot_info_of_lane(si_first, b) : slot_info(p, b));
     if (!si.active) return;
     const int tl = slot_tiles(si);
     const int64_t ooff = (int64_t)b * p.o_s[0] + (int64_t)(g * p.R + row / p.Tq) * p.o_s[1] + (int64_t)(row % p.Tq) * p.o_s[2];

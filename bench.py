@@ -162,7 +162,7 @@ class BatchedDecode(Workload):
     bound = "hbm"
 
     def __init__(self, device, B=64, kv_ctx=32768, len_lo=128, len_hi=32768, swa_every=2, seed=0, name="decode_batched_b64",
-                 heads=H, groups=G, dim=D):
+                 heads=H, groups=G, dim=D, layer_window=None):
         import numpy as np
         import torch
 
@@ -176,6 +176,11 @@ class BatchedDecode(Workload):
         rng = np.random.default_rng(seed)
         self.tds_list = rng.integers(len_lo, len_hi + 1, B).tolist()
         self.win_list = [512 if (swa_every and b % swa_every == 0) else kv_ctx for b in range(B)]
+        # layer_window: a sliding-window layer of the engine -- one window for every slot (ctx_window_size), no per-slot
+        # windows, rings of kv_ctx rows
+        self.layer_window = layer_window
+        if layer_window:
+            self.win_list = [layer_window] * B
         self.n_keys = [min(t, w) for t, w in zip(self.tds_list, self.win_list)]
         self.q = _randn_f16((B, H_, 1, D_), seed + 1, device)
         self.k = _randn_f16((B, G_, kv_ctx, D_), seed + 2, device)
@@ -195,14 +200,17 @@ class BatchedDecode(Workload):
         plan = self.plans.get(kernel_mask)
         if plan is None:
             plan = self.plans[kernel_mask] = self.fa2.plan_flash_attention(
-                self.q, self.k, self.v, self.o, self.tds, self.phase, self.kv_ctx, self.fa2.PHASE_DECODE,
-                scale=SCALE, window_sizes=self.win, workspace=WORKSPACE_OF(self.ws), kernel_mask=kernel_mask,
+                self.q, self.k, self.v, self.o, self.tds, self.phase, self.layer_window or self.kv_ctx, self.fa2.PHASE_DECODE,
+                scale=SCALE, window_sizes=None if self.layer_window else self.win, workspace=WORKSPACE_OF(self.ws),
+                kernel_mask=kernel_mask,
             )
         plan.launch()
 
     def cpu_sample(self):
         from oracle import attention_ref as ar
 
+        if self.layer_window:
+            raise NotImplementedError
         # the whole batch, as many passes as fit in about ten seconds of CPU time (the first pass warms the thread pool)
         q, k, v = self.q.cpu(), self.k.cpu(), self.v.cpu()
         phase = [2] * self.B
@@ -494,6 +502,9 @@ WORKLOADS = {
     "decode_batched": lambda dev: BatchedDecode(dev),
     # head dimension 512 (global-attention layers): 32 sequences, every slot attends its whole history
     "decode_batched_d512": lambda dev: BatchedDecode(dev, B=32, swa_every=0, dim=512, name="decode_batched_b32_d512"),
+    # a sliding-window layer of a decode step: 64 sequences, window 512 in rings of 1023 rows (one kernel, no merge)
+    "decode_swa512": lambda dev: BatchedDecode(dev, kv_ctx=1023, len_lo=1024, len_hi=16384, swa_every=0, layer_window=512,
+                                               name="decode_swa512_b64"),
     "decode_single": lambda dev: SingleDecode(dev),
     "prefill_causal_2048": lambda dev: Prefill(dev, 2048),
     "prefill_causal_4096": lambda dev: Prefill(dev, 4096),  # between the configs: pairs of query tiles cut into key spans

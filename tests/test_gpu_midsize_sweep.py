@@ -1,0 +1,97 @@
+"""Seeded random sweep of mid-size prefill-shaped launches (40 .. 5000 query tokens on 0 .. 20000 tokens of context,
+one to four slots, head dimensions 128 / 256 / 512): the sizes where the launch is split over key splits, key spans or
+pairs of query tiles and the merge kernel takes its wider variants.  Every case runs unsplit, split through a poisoned
+workspace and through the library's static scratch; the three must agree, and sampled rows of each are held against an
+fp64 reference computed on the device (on the unrounded query where use_fp32_dot asks for it).  G4B_TEST_SEED_SHIFT=<k>
+runs other draws.
+"""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ATOL_BF16, ATOL_F16, RTOL_BF16, RTOL_F16, ix
+
+pytestmark = pytest.mark.gpu
+N_CASES = 48
+SHIFT = 100000 * int(os.environ.get("G4B_TEST_SEED_SHIFT", "0"))
+
+
+def draw(rng):
+    D = int(rng.choice([128, 256, 256, 512]))
+    R = int(rng.choice([1, 2, 4, 4, 8]))
+    G = int(rng.choice([1, 2, 2, 4]))
+    Tq = int(rng.choice([rng.integers(40, 400), rng.integers(400, 1500), rng.integers(1500, 5000)]))
+    ctx = int(rng.choice([0, 0, rng.integers(1, 3000), rng.integers(3000, 20000)]))
+    B = int(rng.integers(1, 5))
+    kv = ctx + Tq
+    kv_ctx = kv + int(rng.integers(0, 100))
+    qf32 = rng.random() < 0.3
+    return dict(D=D, R=R, G=G, H=R * G, Tq=Tq, B=B, n_in=int(rng.integers(1, B + 1)), kv=kv, kv_ctx=kv_ctx,
+                W=int(rng.choice([kv_ctx, kv_ctx, max(Tq, int(rng.integers(Tq, kv_ctx + 1)))])),
+                qwin=None if rng.random() < 0.6 else int(rng.choice([64, 256, 512, 1000])),
+                stage=ix.STAGE_FULL if rng.random() < 0.15 else ix.STAGE_CAUSAL, bf16=rng.random() < 0.25, qf32=qf32,
+                dot32=qf32 and rng.random() < 0.6, scale=float(rng.choice([1 / 16, 0.25 / np.sqrt(D)])))
+
+
+@pytest.mark.parametrize("n", range(N_CASES))
+def test_random_midsize_prefill(gpu_device, n):
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(31000 + n + SHIFT)
+    c = draw(rng)
+    print(c, flush=True)
+    B, H, G, R, Tq, D, kv_ctx, W, n_in = c["B"], c["H"], c["G"], c["R"], c["Tq"], c["D"], c["kv_ctx"], c["W"], c["n_in"]
+    cdt = torch.bfloat16 if c["bf16"] else torch.float16
+    qdt = torch.float32 if c["qf32"] else cdt
+    g = torch.Generator(device="cuda").manual_seed(32000 + n + SHIFT)
+    q = torch.randn(B, H, Tq, D, generator=g, device="cuda", dtype=torch.float32).to(qdt)
+    k = torch.randn(B, G, kv_ctx, D, generator=g, device="cuda", dtype=torch.float32).to(cdt)
+    v = torch.randn(B, G, kv_ctx, D, generator=g, device="cuda", dtype=torch.float32).to(cdt)
+    kv = c["kv"]
+    tds_list = [int(rng.choice([kv, max(Tq, kv - int(rng.integers(0, 50))), kv + int(rng.integers(0, 3 * kv_ctx))])) for _ in range(B)]
+    tds = torch.tensor(tds_list, dtype=torch.int32, device="cuda")
+    phases = torch.tensor([1] * n_in + [2] * (B - n_in), dtype=torch.uint8, device="cuda")
+    kw = dict(scale=c["scale"], query_window=c["qwin"], stage=c["stage"], use_fp32_dot=c["dot32"])
+
+    def run(**how):
+        o = torch.full((B, H, Tq, D), 777.0, dtype=qdt, device="cuda")
+        fa2.flash_attention(q, k, v, o, tds, phases, W, 1, **how, **kw)
+        return o
+
+    outs = {"unsplit": run(workspace=False), "static scratch": run()}
+    need = fa2.workspace_bytes(B, H, G, Tq, D)
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        ws.fill_(0xFF)  # reads as NaN in every type
+        outs["workspace"] = run(workspace=ws)
+    torch.cuda.synchronize()
+
+    atol, rtol = (ATOL_BF16, RTOL_BF16) if c["bf16"] else (ATOL_F16, RTOL_F16)
+    rows = sorted(set([0, Tq - 1] + rng.integers(0, Tq, 6).tolist()))
+    for b in range(n_in):
+        win, start = ix.window_size(tds_list[b], W), ix.ring_start(tds_list[b], W, kv_ctx)
+        idx = (torch.arange(win, device="cuda") + start) % kv_ctx
+        for i in rows:
+            lo, hi = ix.visible_range(i, tds_list[b], W, Tq, c["stage"], c["qwin"])
+            for h in range(0, H, max(1, H // 3)):
+                # the query as the kernel takes it: unrounded with use_fp32_dot, else rounded to the cache's type
+                qq = q[b, h, i].double() if (c["dot32"] or not c["qf32"]) else q[b, h, i].to(cdt).double()
+                ref = torch.zeros(D, dtype=torch.float64, device="cuda")
+                if hi > lo:
+                    kk, vv = k[b, h // R][idx[lo:hi]].double(), v[b, h // R][idx[lo:hi]].double()
+                    s = (kk @ qq) * c["scale"]
+                    p = torch.exp(s - s.max())
+                    ref = (p / p.sum()) @ vv
+                for name, o in outs.items():
+                    d = (o[b, h, i].double() - ref).abs()
+                    assert bool(torch.isfinite(o[b, h, i]).all()), (name, b, h, i)
+                    assert bool((d <= atol + rtol * ref.abs()).all()), (name, b, h, i, d.max().item())
+    ref = outs["unsplit"][:n_in].double()
+    tol = (8e-3 if c["bf16"] else 1e-3) + (2e-2 if c["bf16"] else 4e-3) * ref.abs()
+    for name, o in outs.items():
+        assert bool(torch.isfinite(o[:n_in]).all()), name
+        assert bool((o[n_in:] == 777.0).all()), f"{name}: rows of slots that are not in phase were written"
+        assert bool(((o[:n_in].double() - ref).abs() <= tol).all()), f"{name} against unsplit"

@@ -95,3 +95,83 @@ def test_random_midsize_prefill(gpu_device, n):
         assert bool(torch.isfinite(o[:n_in]).all()), name
         assert bool((o[n_in:] == 777.0).all()), f"{name}: rows of slots that are not in phase were written"
         assert bool(((o[:n_in].double() - ref).abs() <= tol).all()), f"{name} against unsplit"
+
+
+def draw_decode(rng):
+    D = int(rng.choice([128, 256, 256, 512]))
+    R = int(rng.choice([1, 2, 4, 4, 8, 16]))
+    G = int(rng.choice([1, 2, 2, 4]))
+    Tq = int(rng.choice([1, 1, 1, 2, 3, 4]))
+    while R * Tq > 16:
+        Tq -= 1
+    kv_ctx = int(rng.choice([rng.integers(40, 600), rng.integers(600, 5000), rng.integers(5000, 20000)]))
+    qf32 = rng.random() < 0.3
+    return dict(D=D, R=R, G=G, H=R * G, Tq=Tq, B=int(rng.choice([1, 2, 5, 17, 33, 64])), kv_ctx=kv_ctx,
+                W=int(rng.choice([kv_ctx, kv_ctx, int(rng.integers(max(Tq, 1), kv_ctx + 1)), min(kv_ctx, 512)])),
+                per_slot=rng.random() < 0.3, bf16=rng.random() < 0.25, qf32=qf32, dot32=qf32 and rng.random() < 0.6,
+                scale=float(rng.choice([1 / 16, 0.25 / np.sqrt(D)])), nw=int(rng.choice([0, 0, 0, 7, 100, 3000])))
+
+
+@pytest.mark.parametrize("n", range(N_CASES))
+def test_random_midsize_decode(gpu_device, n):
+    """Decode-shaped launches of 1 .. 64 slots on rings of 40 .. 20000 rows (empty, filling, full and wrapped slots,
+    slots of other phases, per-slot windows, short windows that take the one-kernel path, worker counts from 7 to 3000):
+    one wave per pair, workers + merge through a poisoned workspace and through the static scratch, all against fp64
+    rows."""
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(41000 + n + SHIFT)
+    c = draw_decode(rng)
+    print(c, flush=True)
+    B, H, G, R, Tq, D, kv_ctx, W = c["B"], c["H"], c["G"], c["R"], c["Tq"], c["D"], c["kv_ctx"], c["W"]
+    win_list = [int(rng.integers(Tq, W + 1)) for _ in range(B)] if c["per_slot"] else None
+    tds_list = [int(rng.choice([0, Tq, int(rng.integers(Tq, W + 1)), W, int(rng.integers(W, 4 * kv_ctx))])) for _ in range(B)]
+    tds_list = [t if t >= Tq or t == 0 else Tq for t in tds_list]
+    ph_list = [2 if rng.random() < 0.85 else int(rng.choice([0, 1])) for _ in range(B)]
+    cdt = torch.bfloat16 if c["bf16"] else torch.float16
+    qdt = torch.float32 if c["qf32"] else cdt
+    g = torch.Generator(device="cuda").manual_seed(42000 + n + SHIFT)
+    q = torch.randn(B, H, Tq, D, generator=g, device="cuda", dtype=torch.float32).to(qdt)
+    k = torch.randn(B, G, kv_ctx, D, generator=g, device="cuda", dtype=torch.float32).to(cdt)
+    v = torch.randn(B, G, kv_ctx, D, generator=g, device="cuda", dtype=torch.float32).to(cdt)
+    tds = torch.tensor(tds_list, dtype=torch.int32, device="cuda")
+    phases = torch.tensor(ph_list, dtype=torch.uint8, device="cuda")
+    win = torch.tensor(win_list, dtype=torch.int32, device="cuda") if win_list else None
+    kw = dict(scale=c["scale"], use_fp32_dot=c["dot32"], window_sizes=win)
+
+    def run(**how):
+        o = torch.full((B, H, Tq, D), 777.0, dtype=qdt, device="cuda")
+        fa2.flash_attention(q, k, v, o, tds, phases, W, 2, **how, **kw)
+        return o
+
+    need = fa2.workspace_bytes(B, H, G, Tq, D, c["nw"])
+    ws = torch.empty(max(16, need), dtype=torch.uint8, device="cuda")
+    ws.fill_(0xFF)
+    outs = {"one wave per pair": run(workspace=False), "workspace": run(workspace=ws, num_workers=c["nw"])}
+    if need <= fa2._native.load().g4b_static_scratch_bytes():
+        outs["static scratch"] = run(workspace="static", num_workers=c["nw"])
+    torch.cuda.synchronize()
+
+    atol, rtol = (ATOL_BF16, RTOL_BF16) if c["bf16"] else (ATOL_F16, RTOL_F16)
+    for b in range(B):
+        if ph_list[b] != 2:
+            for name, o in outs.items():
+                assert bool((o[b] == 777.0).all()), f"{name}: slot {b} is not in phase and was written"
+            continue
+        Wb = win_list[b] if win_list else W
+        wsz, start = ix.window_size(tds_list[b], Wb), ix.ring_start(tds_list[b], Wb, kv_ctx)
+        idx = (torch.arange(wsz, device="cuda") + start) % kv_ctx
+        for i in range(Tq):
+            lo, hi = ix.visible_range(i, tds_list[b], Wb, Tq, ix.STAGE_CAUSAL, None)
+            for h in range(0, H, max(1, H // 3)):
+                qq = q[b, h, i].double() if (c["dot32"] or not c["qf32"]) else q[b, h, i].to(cdt).double()
+                ref = torch.zeros(D, dtype=torch.float64, device="cuda")
+                if hi > lo:
+                    kk, vv = k[b, h // R][idx[lo:hi]].double(), v[b, h // R][idx[lo:hi]].double()
+                    s = (kk @ qq) * c["scale"]
+                    p = torch.exp(s - s.max())
+                    ref = (p / p.sum()) @ vv
+                for name, o in outs.items():
+                    d = (o[b, h, i].double() - ref).abs()
+                    assert bool(torch.isfinite(o[b, h, i]).all()), (name, b, h, i)
+                    assert bool((d <= atol + rtol * ref.abs()).all()), (name, b, h, i, tds_list[b], Wb, d.max().item())

@@ -175,3 +175,64 @@ def test_random_midsize_decode(gpu_device, n):
                     d = (o[b, h, i].double() - ref).abs()
                     assert bool(torch.isfinite(o[b, h, i]).all()), (name, b, h, i)
                     assert bool((d <= atol + rtol * ref.abs()).all()), (name, b, h, i, tds_list[b], Wb, d.max().item())
+
+
+N_MIXED = 36
+
+
+@pytest.mark.parametrize("n", range(N_MIXED))
+def test_random_midsize_mixed_launch(gpu_device, n):
+    """Prefill-phase and decode-phase slots in one launch at mid sizes (chunks of 64 .. 1024 tokens, 2 .. 40 slots, rings
+    up to 20000 rows, both head dimensions) against the two separate launches of the same arguments, which the sweeps
+    above hold against fp64 rows."""
+    from g4b_amd.kernels import fa2
+
+    rng = np.random.default_rng(51000 + n + SHIFT)
+    D = int(rng.choice([256, 512]))
+    R = int(rng.choice([1, 2, 4, 4, 8]))
+    G = int(rng.choice([1, 2, 2, 4]))
+    H = R * G
+    t = int(rng.choice([64, 128, 200, 512, 1024]))
+    td = 1 if R > 8 or rng.random() < 0.7 else 2
+    B = int(rng.choice([2, 3, 9, 33, 40]))
+    kv_ctx = int(rng.choice([rng.integers(t + 8, 3000), rng.integers(3000, 20000)]))
+    W = int(rng.choice([kv_ctx, kv_ctx, int(rng.integers(t, kv_ctx + 1)), max(t, min(kv_ctx, 512))]))
+    phase = [int(rng.choice([1, 2, 2, 2, 2, 0])) for _ in range(B)]
+    phase[int(rng.integers(0, B))] = 1
+    if 2 not in phase:
+        phase[(phase.index(1) + 1) % B] = 2
+    tds = [int(rng.choice([t if p == 1 else td, int(rng.integers(t, max(t, W) + 1)), int(rng.integers(W, 4 * kv_ctx))])) for p in phase]
+    bf16, q_f32 = rng.random() < 0.25, rng.random() < 0.3
+    fp32_dot = q_f32 and rng.random() < 0.5
+    scale = float(rng.choice([1 / 16, 0.25 / np.sqrt(D)]))
+    print(dict(D=D, H=H, G=G, t=t, td=td, B=B, kv_ctx=kv_ctx, W=W, phase=phase, tds=tds, bf16=bf16, q_f32=q_f32, fp32_dot=fp32_dot),
+          flush=True)
+    cdt = torch.bfloat16 if bf16 else torch.float16
+    qdt = torch.float32 if q_f32 else cdt
+    g = torch.Generator(device="cuda").manual_seed(52000 + n + SHIFT)
+    qp = torch.randn(B, H, t, D, generator=g, device="cuda", dtype=torch.float32).to(qdt)
+    qd = torch.randn(B, H, td, D, generator=g, device="cuda", dtype=torch.float32).to(qdt)
+    k = torch.randn(B, G, kv_ctx, D, generator=g, device="cuda", dtype=torch.float32).to(cdt)
+    v = torch.randn(B, G, kv_ctx, D, generator=g, device="cuda", dtype=torch.float32).to(cdt)
+    tds_t = torch.tensor(tds, dtype=torch.int32, device="cuda")
+    ph_t = torch.tensor(phase, dtype=torch.uint8, device="cuda")
+    kw = dict(scale=scale, use_fp32_dot=fp32_dot)
+
+    def fresh(tok):
+        return torch.full((B, H, tok, D), 777.0, dtype=qdt, device="cuda")
+
+    ref_p, ref_d = fresh(t), fresh(td)
+    fa2.flash_attention(qp, k, v, ref_p, tds_t, ph_t, W, 1, workspace=False, **kw)
+    fa2.flash_attention(qd, k, v, ref_d, tds_t, ph_t, W, 2, workspace=False, **kw)
+    nbytes = fa2.mixed_workspace_bytes(B, H, G, t, td, D, kv_ctx, W)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    for how in ("workspace", "no workspace"):
+        ws.fill_(0xFF)
+        op, od = fresh(t), fresh(td)
+        fa2.flash_attention(qp, k, v, op, tds_t, ph_t, W, 1, decode_q=qd, decode_o=od, workspace=ws if how == "workspace" else False, **kw)
+        torch.cuda.synchronize()
+        for got, ref, what in ((op, ref_p, "chunk"), (od, ref_d, "decode")):
+            assert bool(torch.isfinite(got).all()), (how, what)
+            d = (got.double() - ref.double()).abs()
+            tol = (8e-3 if bf16 else 1e-3) + (2e-2 if bf16 else 4e-3) * ref.double().abs()
+            assert bool((d <= tol).all()), (how, what, d.max().item())

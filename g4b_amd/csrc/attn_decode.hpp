@@ -101,7 +101,11 @@ G4B_DEV float pick(const f4& c, int e, int cls) {
 //
 // QS: the query is wider than the cache type and enters the first product as two operands (rounded value, rounding
 // error), so the scores see the unrounded query.
-template <int D, int CL, class T, int DH, bool QS>
+//
+// PF: key tiles whose loads are in flight ahead of the arithmetic.  One leaves a streaming worker's registers to its
+// 32 KB tile and is all that a launch of a thousand workers needs; in a mixed launch, where the stream has part of the
+// chip and the kernel's register budget is that of the prefill body anyway, a worker asks for two tiles at a time.
+template <int D, int CL, class T, int DH, bool QS, int PF = 1>
 G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int bb, int g, int t0, int t1, int tlb,
                             float* xch, float* lds_part = nullptr) {
     constexpr int DL = D / DH;         // columns this wave owns
@@ -164,24 +168,26 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
         return (uint32_t)r * ROWB;
     };
 
-    u4 kreg[NT][NC];
-    u4 vreg[DC][8];
-    auto load_k = [&](int t) {
+    u4 kreg[PF][NT][NC];
+    u4 vreg[PF][DC][8];
+    auto load_k = [&](int t, auto buf) {
         const int jb = si.klo + t * DEC_TILE;
 #pragma unroll
         for (int tau = 0; tau < NT; ++tau) {
             const uint32_t ro = key_off(jb + tau * KT + m16 / CL);
 #pragma unroll
-            for (int c = 0; c < NC; ++c) kreg[tau][c] = G4B_DEC_LD(kbase, ro + (uint32_t)(cls + CL * g4 + 4 * CL * c) * 16u);
+            for (int c = 0; c < NC; ++c)
+                kreg[decltype(buf)::value][tau][c] = G4B_DEC_LD(kbase, ro + (uint32_t)(cls + CL * g4 + 4 * CL * c) * 16u);
         }
     };
-    auto load_v = [&](int t) {
+    auto load_v = [&](int t, auto buf) {
         const int jb = si.klo + t * DEC_TILE;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const uint32_t ro = key_off(jb + (s / E) * KT + g4 * E + (s % E));
 #pragma unroll
-            for (int dc = 0; dc < DC; ++dc) vreg[dc][s] = G4B_DEC_LD(vbase, ro + (uint32_t)(m16 + 16 * dc) * 16u);
+            for (int dc = 0; dc < DC; ++dc)
+                vreg[decltype(buf)::value][dc][s] = G4B_DEC_LD(vbase, ro + (uint32_t)(m16 + 16 * dc) * 16u);
         }
     };
 
@@ -190,10 +196,19 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
 #pragma unroll
     for (int i = 0; i < DC * 8; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
 
-    load_k(t0);
-    load_v(t0);
+    static_assert(PF == 1 || PF == 2, "one or two tiles ahead");
+    load_k(t0, std::integral_constant<int, 0>{});
+    load_v(t0, std::integral_constant<int, 0>{});
+    if constexpr (PF == 2) {
+        if (t0 + 1 < t1) {
+            load_k(t0 + 1, std::integral_constant<int, 1>{});
+            load_v(t0 + 1, std::integral_constant<int, 1>{});
+        }
+    }
     if constexpr (DH > 1) __syncthreads();  // the exchange buffers of the previous segment are free
-    for (int t = t0; t < t1; ++t) {
+    // one key tile: the tile in buffer `buf`, whose next occupant (tile t + PF) is asked for as soon as the buffer is read
+    auto tile = [&](int t, auto buf) {
+        constexpr int BUF = decltype(buf)::value;
         const int jb = si.klo + t * DEC_TILE;
         // ---- S^T = K Q^T -------------------------------------------------------
         float sc[8];
@@ -202,8 +217,8 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
             f4 c4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                if constexpr (QS) c4 = T::mfma16(kreg[tau][c], qf_lo[c], c4);
-                c4 = T::mfma16(kreg[tau][c], qf[c], c4);
+                if constexpr (QS) c4 = T::mfma16(kreg[BUF][tau][c], qf_lo[c], c4);
+                c4 = T::mfma16(kreg[BUF][tau][c], qf[c], c4);
             }
 #pragma unroll
             for (int e = 0; e < E; ++e) {
@@ -213,7 +228,7 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
                 sc[tau * E + e] = x * p.c;
             }
         }
-        if (t + 1 < t1) load_k(t + 1);
+        if (t + PF < t1) load_k(t + PF, buf);
         if constexpr (DH > 1) {
             // add the other waves' partial dot products; buffers alternate so one barrier per tile is enough
             float* xb = xch + (t & 1) * (DH * 8 * 64);
@@ -260,11 +275,17 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
             u4 vt[8];
-            transpose8x8_b16(vreg[dc], vt);
+            transpose8x8_b16(vreg[BUF][dc], vt);
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) acc[dc * 8 + jj] = T::mfma16(vt[jj], pf, acc[dc * 8 + jj]);
         }
-        if (t + 1 < t1) load_v(t + 1);
+        if (t + PF < t1) load_v(t + PF, buf);
+    };
+    for (int t = t0; t < t1; t += PF) {
+        tile(t, std::integral_constant<int, 0>{});
+        if constexpr (PF == 2) {
+            if (t + 1 < t1) tile(t + 1, std::integral_constant<int, 1>{});
+        }
     }
 
     // ---- epilogue -----------------------------------------------------------------
@@ -311,7 +332,7 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
 
 // Worker w of a launch: its share of the flat tile list.  Called by every wave of the worker (DH of them); xch is the
 // worker's exchange buffer when DH > 1.
-template <int D, int CL, class T, int DH, bool QS>
+template <int D, int CL, class T, int DH, bool QS, int PF = 1>
 G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
     const int lane = threadIdx.x & 63;  // every wave of the worker does the same bookkeeping
     const int B = p.B, G = p.G;
@@ -323,7 +344,7 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
         const SlotInfo si = slot_info(p, bb);
         const int tlb = slot_tiles(si);
         if (tlb > 0) {
-            decode_segment<D, CL, T, DH, QS>(p, si, w, bb, g, 0, tlb, tlb, xch);
+            decode_segment<D, CL, T, DH, QS, PF>(p, si, w, bb, g, 0, tlb, tlb, xch);
         } else if (si.active && (DH == 1 || threadIdx.x < 64)) {  // one wave of the worker
             // in-phase slot without any visible key: defined as zeros (no merge kernel runs on this path)
             const int NR = p.R * p.Tq;
@@ -349,7 +370,7 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
             const int64_t fs = (int64_t)g * tlb;
             const int t0 = (int)(max(ws, fs) - fs);
             const int t1 = (int)(min(we, fs + tlb) - fs);
-            if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, si, w, 0, g, t0, t1, tlb, xch);
+            if (t1 > t0) decode_segment<D, CL, T, DH, QS, PF>(p, si, w, 0, g, t0, t1, tlb, xch);
         }
         return;
     }
@@ -395,7 +416,7 @@ G4B_DEV void decode_worker_body(const AttnParams& p, int w, float* xch) {
                 const int64_t fs = (int64_t)ex + (int64_t)g * tlb;
                 const int t0 = (int)(max(ws, fs) - fs);
                 const int t1 = (int)(min(we, fs + tlb) - fs);
-                if (t1 > t0) decode_segment<D, CL, T, DH, QS>(p, si, w, bb, g, t0, t1, tlb, xch);
+                if (t1 > t0) decode_segment<D, CL, T, DH, QS, PF>(p, si, w, bb, g, t0, t1, tlb, xch);
             }
         }
         carry += __builtin_amdgcn_readlane(incl, 63);

@@ -22,6 +22,11 @@
 
 namespace g4b {
 
+// Key tiles that a decode worker of a head-dimension-512 mixed launch keeps in flight: its four waves own 128 columns
+// each and so half the bytes per tile of a streaming worker elsewhere (the 35-layer step with 512-wide global layers
+// 5.44 -> 5.30 ms; at head dimension 256, where a worker is one wave with a whole tile, two measured the same as one).
+constexpr int MIXED_DECODE_PF = 2;
+
 template <int D, int CL, class T, bool QS>
 __global__ __launch_bounds__(256) void attn_mixed_kernel(const AttnParams pp, const AttnParams pd, const MixedPlan mp) {
     extern __shared__ __align__(16) char smem[];
@@ -37,7 +42,7 @@ __global__ __launch_bounds__(256) void attn_mixed_kernel(const AttnParams pp, co
     const int d = j * 8 + x;
     if (d >= mp.nd_blocks) return;
     if constexpr (D == 512) {
-        decode_worker_body<D, CL, T, 4, QS>(pd, d, reinterpret_cast<float*>(smem));
+        decode_worker_body<D, CL, T, 4, QS, MIXED_DECODE_PF>(pd, d, reinterpret_cast<float*>(smem));
     } else {
         if (mp.pair_path) {
             decode_pair_body<D, CL, T, QS>(pd, d, reinterpret_cast<float*>(smem));

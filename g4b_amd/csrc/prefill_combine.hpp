@@ -32,7 +32,9 @@ G4B_DEV void prefill_combine_rows(const AttnParams& p, int a_idx, int b, int h, 
     const char* const o_base = reinterpret_cast<const char*>(p.part_o) + row_base * (D * 2);
     const char* const ml_base = reinterpret_cast<const char*>(p.part_ml) + row_base * 8;
     int t[PASSES];
-    uint32_t o_off[PASSES], ml_off[PASSES];  // of a lane's row (clamped to the last one: loaded twice, stored once)
+    // byte offsets of a lane's row (clamped to the last one: loaded twice, stored once); 32 bits are plenty: only
+    // launches whose query tiles do not fill the chip are split (api.hip::prefill_split_slots), a few thousand tokens
+    uint32_t o_off[PASSES], ml_off[PASSES];
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
         t[pass] = tb * ROWS + pass * RPP + r_in;

@@ -268,8 +268,11 @@ G4B_DEV void decode_segment(const AttnParams& p, const SlotInfo& si, int w, int 
         l_run = l_run * alpha + psum;
         m_run = m_new;
         const u4 pf = {T::pack2(ps[0], ps[1]), T::pack2(ps[2], ps[3]), T::pack2(ps[4], ps[5]), T::pack2(ps[6], ps[7])};
+        // (nothing to rescale on the first tile, and on most later ones no row's maximum has moved)
+        if (t > t0 && __any(alpha != 1.f)) {
 #pragma unroll
-        for (int i = 0; i < DC * 8; ++i) acc[i] *= alpha;
+            for (int i = 0; i < DC * 8; ++i) acc[i] *= alpha;
+        }
 
         // ---- O^T += V^T P ------------------------------------------------------
 #pragma unroll
